@@ -1,0 +1,196 @@
+"""ctypes binding of libspattn_hip.so (declared in include/spattn_hip.h).
+
+Tensors are torch device tensors used only as owners of HBM; the calls pass raw
+pointers and sizes.  There is no fallback: a missing library raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+from pathlib import Path
+
+import torch
+
+_LIB_PATH = Path(__file__).resolve().parent / "libspattn_hip.so"
+_lib = None
+
+_c_int, _c_float, _c_void_p = ctypes.c_int, ctypes.c_float, ctypes.c_void_p
+
+# name -> argtypes, for every symbol the header declares
+_SIGNATURES = {
+    # the reference's binding surface (void return)
+    "attn_fwd_wg_impl": (None, [_c_void_p] * 4 + [_c_int] * 4),
+    "attn_sparse_fwd_wg_impl": (None, [_c_void_p] * 6 + [_c_int] * 5),
+    "allindex_mask_impl": (None, [_c_void_p] * 2 + [_c_int] * 4),
+    "attn_maxq_denom_impl": (None, [_c_void_p] * 6 + [_c_int] * 4),
+    "maxq_denom_impl": (None, [_c_void_p] * 4 + [_c_int] * 4),
+    "booleanmask_128_impl": (None, [_c_void_p, _c_float, _c_int] + [_c_void_p] * 4 + [_c_int] * 4),
+    "booleanmask_to_indexmask_impl": (None, [_c_void_p] * 3 + [_c_int] * 5),
+    # extended entry points (status return)
+    "spattn_full_attn": (_c_int, [_c_void_p] * 5 + [_c_int] * 5 + [_c_float, _c_void_p]),
+    "spattn_sp_attn": (_c_int, [_c_void_p] * 7 + [_c_int] * 7 + [_c_float, _c_void_p]),
+    "spattn_sp_attn_blocks": (_c_int, [_c_void_p] * 7 + [_c_int] * 7 + [_c_float, _c_void_p]),
+    "spattn_all_index_mask": (_c_int, [_c_void_p] * 2 + [_c_int] * 5 + [_c_void_p]),
+    "spattn_fullattn_maxq_denom": (_c_int, [_c_void_p] * 6 + [_c_int] * 5 + [_c_float, _c_void_p]),
+    "spattn_maxq_denom": (_c_int, [_c_void_p] * 4 + [_c_int] * 5 + [_c_float, _c_void_p]),
+    "spattn_booleanmask_128": (_c_int, [_c_void_p, _c_float, _c_int] + [_c_void_p] * 4 + [_c_int] * 5 + [_c_float, _c_void_p]),
+    "spattn_booleanmask_to_indexmask": (_c_int, [_c_void_p] * 3 + [_c_int] * 5 + [_c_void_p]),
+    "spattn_last_status": (_c_int, []),
+    "spattn_status_string": (ctypes.c_char_p, [_c_int]),
+    "spattn_version": (_c_int, []),
+}
+
+
+class SpattnError(RuntimeError):
+    def __init__(self, status: int, text: str):
+        super().__init__("spattn status %d: %s" % (status, text))
+        self.status = status
+
+
+def lib_path() -> Path:
+    return _LIB_PATH
+
+
+def exported_symbols():
+    return sorted(_SIGNATURES)
+
+
+def load() -> ctypes.CDLL:
+    """Load libspattn_hip.so; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not _LIB_PATH.exists():
+            raise RuntimeError(
+                "%s is missing: build it with `python -m fgattn_tk_cuda_amd.build --lib-only`" % _LIB_PATH)
+        lib = ctypes.CDLL(str(_LIB_PATH))
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def _check(status: int) -> None:
+    if status != 0:
+        raise SpattnError(status, load().spattn_status_string(status).decode())
+
+
+def _ptr(t, dtype=None):
+    if t is None:
+        return None
+    if not t.is_cuda:
+        raise ValueError("expected a device tensor")
+    if not t.is_contiguous():
+        raise ValueError("expected a contiguous tensor")
+    if dtype is not None and t.dtype != dtype:
+        raise ValueError("expected dtype %s, got %s" % (dtype, t.dtype))
+    return t.data_ptr()
+
+
+def _stream(stream=None):
+    if stream is None:
+        stream = torch.cuda.current_stream()
+    return stream.cuda_stream
+
+
+def _bhsd(q):
+    if q.dim() != 4:
+        raise ValueError("q must be [B,H,S,D]")
+    return tuple(int(x) for x in q.shape)
+
+
+bf16, i32, f32 = torch.bfloat16, torch.int32, torch.float32
+
+
+def full_attn(o, q, k, v, *, lse=None, kv_len=0, scale=0.0, stream=None):
+    B, H, S, D = _bhsd(q)
+    _check(load().spattn_full_attn(_ptr(o, bf16), _ptr(lse, f32), _ptr(q, bf16), _ptr(k, bf16), _ptr(v, bf16),
+                                   B, H, S, D, kv_len, scale, _stream(stream)))
+
+
+def sp_attn(o, q, k, v, kv_indices, kv_num_indices, *, lse=None, qblk=None, kv_len=0, scale=0.0, stream=None):
+    """Token-list sparse attention.  qblk defaults to the value implied by kv_indices.shape[2]."""
+    B, H, S, D = _bhsd(q)
+    if kv_indices.dim() != 4:
+        raise ValueError("kv_indices must be [B,H,SB,mask_stride]")
+    if qblk is None:
+        qblk = infer_qblk(S, int(kv_indices.shape[2]))
+    if kv_num_indices.numel() != B * H * int(kv_indices.shape[2]):
+        raise ValueError("kv_num_indices must have B*H*SB entries")
+    _check(load().spattn_sp_attn(_ptr(o, bf16), _ptr(lse, f32), _ptr(q, bf16), _ptr(k, bf16), _ptr(v, bf16),
+                                 _ptr(kv_indices, i32), _ptr(kv_num_indices, i32), int(kv_indices.shape[3]), qblk,
+                                 B, H, S, D, kv_len, scale, _stream(stream)))
+
+
+def sp_attn_blocks(o, q, k, v, blk_indices, blk_counts, *, lse=None, qblk=None, kv_len=0, scale=0.0, stream=None):
+    """Block-list sparse attention over 64-key blocks."""
+    B, H, S, D = _bhsd(q)
+    if blk_indices.dim() != 4:
+        raise ValueError("blk_indices must be [B,H,SB,max_blocks]")
+    if qblk is None:
+        qblk = infer_qblk(S, int(blk_indices.shape[2]))
+    if blk_counts.numel() != B * H * int(blk_indices.shape[2]):
+        raise ValueError("blk_counts must have B*H*SB entries")
+    _check(load().spattn_sp_attn_blocks(_ptr(o, bf16), _ptr(lse, f32), _ptr(q, bf16), _ptr(k, bf16), _ptr(v, bf16),
+                                        _ptr(blk_indices, i32), _ptr(blk_counts, i32), int(blk_indices.shape[3]),
+                                        qblk, B, H, S, D, kv_len, scale, _stream(stream)))
+
+
+def all_index_mask(kv_indices, kv_num_indices, batch, heads, seqblocks, seq, *, stream=None):
+    _check(load().spattn_all_index_mask(_ptr(kv_indices, i32), _ptr(kv_num_indices, i32), batch, heads, seqblocks, seq,
+                                        int(kv_indices.shape[-1]), _stream(stream)))
+
+
+def fullattn_maxq_denom(o, max_q, denom, q, k, v, *, kv_len=0, scale=0.0, stream=None):
+    B, H, S, D = _bhsd(q)
+    _need_padded(max_q, denom, B, H, S)
+    _check(load().spattn_fullattn_maxq_denom(_ptr(o, bf16), _ptr(max_q, f32), _ptr(denom, f32), _ptr(q, bf16),
+                                             _ptr(k, bf16), _ptr(v, bf16), B, H, S, D, kv_len, scale, _stream(stream)))
+
+
+def maxq_denom(max_q, denom, q, k, *, kv_len=0, scale=0.0, stream=None):
+    B, H, S, D = _bhsd(q)
+    _need_padded(max_q, denom, B, H, S)
+    _check(load().spattn_maxq_denom(_ptr(max_q, f32), _ptr(denom, f32), _ptr(q, bf16), _ptr(k, bf16), B, H, S, D,
+                                    kv_len, scale, _stream(stream)))
+
+
+def booleanmask_128(booleanmask, max_q, denom, q, k, threshold, *, kv_len=0, scale=0.0, stream=None):
+    B, H, S, D = _bhsd(q)
+    _need_padded(max_q, denom, B, H, S)
+    if booleanmask.dim() != 4 or int(booleanmask.shape[2]) != (S + 127) // 128:
+        raise ValueError("booleanmask must be [B,H,ceil(S/128),mask_stride]")
+    _check(load().spattn_booleanmask_128(_ptr(booleanmask, i32), float(threshold), int(booleanmask.shape[3]),
+                                         _ptr(max_q, f32), _ptr(denom, f32), _ptr(q, bf16), _ptr(k, bf16), B, H, S, D,
+                                         kv_len, scale, _stream(stream)))
+
+
+def booleanmask_to_indexmask(kv_indices, kv_num_indices, booleanmask, seq, *, stream=None):
+    if booleanmask.dim() != 4:
+        raise ValueError("booleanmask must be [B,H,SB,mask_stride]")
+    B, H, SB, MS = (int(x) for x in booleanmask.shape)
+    if tuple(kv_indices.shape) != (B, H, SB, MS) or kv_num_indices.numel() != B * H * SB:
+        raise ValueError("kv_indices / kv_num_indices do not match booleanmask")
+    _check(load().spattn_booleanmask_to_indexmask(_ptr(kv_indices, i32), _ptr(kv_num_indices, i32),
+                                                  _ptr(booleanmask, i32), B, H, int(seq), SB, MS, _stream(stream)))
+
+
+def infer_qblk(seq: int, seqblocks: int) -> int:
+    """Rows per q-block from the number of lists per head; 128 (the reference's) wins a tie."""
+    if seqblocks == (seq + 127) // 128:
+        return 128
+    if seqblocks == (seq + 63) // 64:
+        return 64
+    raise ValueError("index tensor has %d q-blocks; expected ceil(S/128) or ceil(S/64)" % seqblocks)
+
+
+def _need_padded(max_q, denom, B, H, S):
+    sp = 128 * ((S + 127) // 128)
+    for t in (max_q, denom):
+        if t.numel() != B * H * sp:
+            raise ValueError("max_q/denom must hold B*H*%d floats" % sp)
+
+
+def default_scale(D: int) -> float:
+    return 1.0 / math.sqrt(D)

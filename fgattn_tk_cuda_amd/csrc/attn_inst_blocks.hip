@@ -1,0 +1,15 @@
+// Block-list sparse attention instantiations (64-key blocks).
+#include "attn_fwd.h"
+#include "dispatch.h"
+
+namespace spattn {
+
+hipError_t run_attn_blocks(const AttnParams& p, int D, int qblk, hipStream_t stream) {
+  if (D == 128 && qblk == 128) return launch_attn_fwd<128, 128, KV_BLOCKS, true, false>(p, stream);
+  if (D == 128 && qblk == 64) return launch_attn_fwd<128, 64, KV_BLOCKS, true, false>(p, stream);
+  if (D == 64 && qblk == 128) return launch_attn_fwd<64, 128, KV_BLOCKS, true, false>(p, stream);
+  if (D == 64 && qblk == 64) return launch_attn_fwd<64, 64, KV_BLOCKS, true, false>(p, stream);
+  return hipErrorInvalidValue;
+}
+
+}  // namespace spattn

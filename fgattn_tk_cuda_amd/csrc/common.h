@@ -1,0 +1,70 @@
+// Shared declarations for the gfx950 sparse-attention kernels.
+// Wave = 64 lanes; all matrix work uses v_mfma_f32_32x32x16_bf16.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace spattn {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// How the key rows of one 64-key tile are found.
+enum KvMode : int {
+  KV_DENSE = 0,   // tile t = rows 64t .. 64t+63, up to kv_len
+  KV_TOKENS = 1,  // tile t = rows idx[64t .. 64t+63] of a per-q-block token list
+  KV_BLOCKS = 2,  // tile t = rows 64*blk[t] .. 64*blk[t]+63 of a per-q-block block list
+};
+
+struct AttnParams {
+  const uint16_t* q;
+  const uint16_t* k;
+  const uint16_t* v;
+  uint16_t* o;        // bf16 [B,H,S,D]
+  float* lse;         // optional fp32 [B,H,S], natural log
+  float* max_q;       // optional fp32 [B,H,1,Sp], raw (unscaled) row max
+  float* denom;       // optional fp32 [B,H,1,Sp]
+  const int* idx;     // [B,H,SBq,idx_stride] token ids or block ids
+  const int* cnt;     // [B*H*SBq]
+  int idx_stride;
+  int B, H, S;
+  int kv_len;         // keys with row >= kv_len never contribute
+  int Sp;             // row stride of max_q / denom
+  int nqblk;          // q-blocks per head
+  float scale;        // softmax scale
+  float sf;           // log2(e) * scale
+};
+
+__device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  f32x2 f = {lo, hi};
+  bf16x2 b = __builtin_convertvector(f, bf16x2);   // v_cvt_pk_bf16_f32, round to nearest even
+  return __builtin_bit_cast(uint32_t, b);
+}
+
+// Value held by lane ^ 32.
+__device__ __forceinline__ float xor32(float x) { return __shfl_xor(x, 32, 64); }
+
+// WGs are dealt to the 8 XCDs round-robin by launch order; give each XCD one
+// contiguous range of logical work ids so that neighbouring q-blocks of a head
+// share that XCD's L2.
+__device__ __forceinline__ int xcd_remap(int wg, int total) {
+  constexpr int kXcd = 8;
+  int per = total / kXcd;
+  int lim = per * kXcd;
+  if (wg >= lim) return wg;
+  return (wg % kXcd) * per + wg / kXcd;
+}
+
+}  // namespace spattn

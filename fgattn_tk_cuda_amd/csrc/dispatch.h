@@ -1,0 +1,20 @@
+// Host-side entry points of the kernel translation units (internal, C++).
+#pragma once
+#include "common.h"
+
+namespace spattn {
+
+// attn_inst_tokens.hip / attn_inst_blocks.hip / attn_inst_dense.hip
+hipError_t run_attn_tokens(const AttnParams& p, int D, int qblk, hipStream_t stream);
+hipError_t run_attn_blocks(const AttnParams& p, int D, int qblk, hipStream_t stream);
+hipError_t run_attn_dense(const AttnParams& p, int D, bool has_v, bool stats, hipStream_t stream);
+
+// mask_kernels.hip
+hipError_t run_booleanmask(int* mask, float thresh, int mask_stride, const float* max_q, const float* denom,
+                           const uint16_t* q, const uint16_t* k, int B, int H, int S, int D, int kv_len, float scale,
+                           hipStream_t stream);
+hipError_t run_compact(int* kv_indices, int* kv_num, const int* mask, int rows, int mask_stride, int kv_len,
+                       hipStream_t stream);
+hipError_t run_all_index(int* kv_indices, int* kv_num, int rows, int mask_stride, int seq, hipStream_t stream);
+
+}  // namespace spattn

@@ -1,0 +1,234 @@
+// Threshold-mask pre-pass kernels for gfx950:
+//   booleanmask_128          - QK^T sweep -> per-(q-block, key) vote counts
+//   booleanmask_to_indexmask - vote mask -> ascending key-index lists (HBM-bound stream)
+//   all_index_mask           - identity lists
+#include "common.h"
+#include "dispatch.h"
+
+namespace spattn {
+
+// ------------------------------------------------------------------------------------
+// booleanmask_128.  Reference: include/mask_utils.cuh:131-243.  For q-block I (128 rows)
+// and key c the reference counts the 16-row groups W of I with
+//   max_{r in W} exp2((s[r,c] - max_q[r]) * sf) / denom[r] > thresh        (:231-238)
+// Here the test is done in the log2 domain, which is the same predicate:
+//   max_{r in W} (s[r,c] * sf - (max_q[r] * sf + log2 denom[r])) > log2 thresh.
+// Pad rows carry denom = -inf (include/maxq_denom.cuh:202-205) and never vote.
+//
+// One workgroup per q-block; the 128 x D query tile sits in LDS (16-byte chunks
+// XOR-swizzled by row) and is the A operand.  Each wave walks its own 32-key blocks: the
+// K^T operand goes HBM -> registers with no staging and no barrier, the accumulator of
+// lane (n, g) holds key n against 64 of the 128 query rows, and one exchange with lane
+// n^32 finishes the 8 votes of that key.  The vote count is stored, not accumulated.
+// ------------------------------------------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(256, 2) void booleanmask_kernel(int* __restrict__ mask, const float* __restrict__ max_q,
+                                                              const float* __restrict__ denom,
+                                                              const uint16_t* __restrict__ q,
+                                                              const uint16_t* __restrict__ k, float log2_thresh,
+                                                              int mask_stride, int HB, int S, int kv_len, int Sp,
+                                                              int SB, float sf) {
+  constexpr int NT = D / 16;
+  constexpr int CPR = D / 8;
+  __shared__ __attribute__((aligned(16))) unsigned char qs[128 * D * 2];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int ln = lane & 31;
+  const int g = lane >> 5;
+  const int total = SB * HB;
+  const int wg = xcd_remap(blockIdx.x, total);
+  const int qb = wg % SB;
+  const int bh = wg / SB;
+  const size_t head_off = (size_t)bh * S * D;
+  const uint16_t* qh = q + head_off;
+  const uint16_t* kh = k + head_off;
+
+  // Query tile -> LDS; rows past S are zero.
+  for (int ch = tid; ch < 128 * CPR; ch += 256) {
+    const int r = ch / CPR, c = ch % CPR;
+    const int row = qb * 128 + r;
+    u32x4 val = {0, 0, 0, 0};
+    if (row < S) val = *reinterpret_cast<const u32x4*>(qh + (size_t)row * D + 8 * c);
+    *reinterpret_cast<u32x4*>(qs + r * (D * 2) + ((c ^ (r & (CPR - 1))) << 4)) = val;
+  }
+
+  // Per-row offsets; register 4j+i of block mb is query row 32mb + 8j + 4g + i.
+  float coff[4][16];
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = qb * 128 + 32 * mb + 8 * (r >> 2) + 4 * g + (r & 3);
+      float c = __builtin_huge_valf();
+      if (row < S) {
+        const float mq = max_q[(size_t)bh * Sp + row];
+        const float dn = denom[(size_t)bh * Sp + row];
+        if (dn > 0.f) c = mq * sf + __log2f(dn);
+      }
+      coff[mb][r] = c;
+    }
+  __syncthreads();
+
+  int* mrow = mask + ((size_t)bh * SB + qb) * mask_stride;
+  const int nkb = (mask_stride + 31) >> 5;
+
+  auto load_keys = [&](int kb, u32x4 (&kf)[NT]) {
+    const int key = kb * 32 + ln;
+    const bool ok = kb < nkb && key < kv_len;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const u32x4 z = {0, 0, 0, 0};
+      kf[t] = ok ? *reinterpret_cast<const u32x4*>(kh + (size_t)key * D + 16 * t + 8 * g) : z;
+    }
+  };
+
+  u32x4 kf[NT], kn[NT];
+  load_keys(wave, kf);
+  for (int kb = wave; kb < nkb; kb += 4) {
+    load_keys(kb + 4, kn);
+    unsigned votes = 0;
+    if (kb * 32 < kv_len) {   // wave-uniform
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb) {
+        f32x16 s;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[r] = 0.f;
+        const int qr = 32 * mb + ln;
+        const unsigned char* qrp = qs + qr * (D * 2);
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+          const u32x4 a = *reinterpret_cast<const u32x4*>(qrp + (((2 * t + g) ^ (qr & (CPR - 1))) << 4));
+          s = mfma32(a, kf[t], s);
+        }
+        float w0 = -__builtin_huge_valf(), w1 = -__builtin_huge_valf();
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+          w0 = fmaxf(w0, __builtin_fmaf(s[r], sf, -coff[mb][r]));
+          w1 = fmaxf(w1, __builtin_fmaf(s[8 + r], sf, -coff[mb][8 + r]));
+        }
+        votes |= (w0 > log2_thresh ? 1u : 0u) << (2 * mb);
+        votes |= (w1 > log2_thresh ? 1u : 0u) << (2 * mb + 1);
+      }
+    }
+    // A 16-row group is split over lanes n and n^32: it votes if either half does.
+    votes |= (unsigned)__shfl_xor((int)votes, 32, 64);
+    const int key = kb * 32 + ln;
+    if (g == 0 && key < mask_stride) mrow[key] = (key < kv_len) ? __popc(votes) : 0;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) kf[t] = kn[t];
+  }
+}
+
+hipError_t run_booleanmask(int* mask, float thresh, int mask_stride, const float* max_q, const float* denom,
+                           const uint16_t* q, const uint16_t* k, int B, int H, int S, int D, int kv_len, float scale,
+                           hipStream_t stream) {
+  const int SB = (S + 127) / 128;
+  const int Sp = SB * 128;
+  const float sf = kLog2e * scale;
+  const float lt = thresh > 0.f ? log2f(thresh) : -__builtin_huge_valf();
+  const int total = SB * H * B;
+  if (total <= 0) return hipSuccess;
+  if (D == 128) {
+    hipLaunchKernelGGL(booleanmask_kernel<128>, dim3(total, 1, 1), dim3(256), 0, stream, mask, max_q, denom, q, k, lt,
+                       mask_stride, H * B, S, kv_len, Sp, SB, sf);
+  } else {
+    hipLaunchKernelGGL(booleanmask_kernel<64>, dim3(total, 1, 1), dim3(256), 0, stream, mask, max_q, denom, q, k, lt,
+                       mask_stride, H * B, S, kv_len, Sp, SB, sf);
+  }
+  return hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------------
+// booleanmask_to_indexmask.  Reference: include/mask_utils.cuh:273-302 - for each
+// (b,h,q-block) row: count = #{c < kv_len : mask[c] > 0}, list = those c, entries past the
+// count keep the caller's fill.  The reference appends through one global atomic per key
+// (order undefined); here one wave owns one row, reads it as 16-byte vectors, ranks every
+// kept key with wave ballots and writes the list in ascending order - no atomics, no LDS,
+// no barrier, and the result is deterministic.  The kernel is a pure HBM stream:
+// 4 bytes read per mask entry, 4 bytes written per kept key.
+// ------------------------------------------------------------------------------------
+constexpr int kCompactUnroll = 8;   // 16-byte loads in flight per lane
+
+__global__ __launch_bounds__(256) void compact_kernel(int* __restrict__ kv_indices, int* __restrict__ kv_num,
+                                                      const int* __restrict__ mask, int rows, int mask_stride,
+                                                      int kv_len) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int* __restrict__ src = mask + (size_t)row * mask_stride;
+  int* __restrict__ dst = kv_indices + (size_t)row * mask_stride;
+  const int lim = kv_len < mask_stride ? kv_len : mask_stride;
+  int base = 0;
+  constexpr int kSpan = 64 * 4 * kCompactUnroll;   // ints per wave iteration
+  for (int c0 = 0; c0 < lim; c0 += kSpan) {
+    i32x4 val[kCompactUnroll];
+#pragma unroll
+    for (int u = 0; u < kCompactUnroll; ++u) {
+      const int e0 = c0 + u * 256 + 4 * lane;
+      const i32x4 z = {0, 0, 0, 0};
+      val[u] = (e0 < lim) ? __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(src + e0)) : z;
+    }
+#pragma unroll
+    for (int u = 0; u < kCompactUnroll; ++u) {
+      const int e0 = c0 + u * 256 + 4 * lane;
+      bool f[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) f[i] = (e0 + i < lim) && (val[u][i] > 0);
+      const unsigned long long b0 = __ballot(f[0]), b1 = __ballot(f[1]), b2 = __ballot(f[2]), b3 = __ballot(f[3]);
+      if ((b0 | b1 | b2 | b3) == 0ull) continue;
+      // keys of lower lanes come first, then this lane's own lower keys
+      int pos = base;
+      pos = __builtin_amdgcn_mbcnt_hi((unsigned)(b0 >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)b0, pos));
+      pos = __builtin_amdgcn_mbcnt_hi((unsigned)(b1 >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)b1, pos));
+      pos = __builtin_amdgcn_mbcnt_hi((unsigned)(b2 >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)b2, pos));
+      pos = __builtin_amdgcn_mbcnt_hi((unsigned)(b3 >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)b3, pos));
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (f[i]) dst[pos] = e0 + i;
+        pos += f[i] ? 1 : 0;
+      }
+      base += __popcll(b0) + __popcll(b1) + __popcll(b2) + __popcll(b3);
+    }
+  }
+  if (lane == 0) kv_num[row] = base;
+}
+
+hipError_t run_compact(int* kv_indices, int* kv_num, const int* mask, int rows, int mask_stride, int kv_len,
+                       hipStream_t stream) {
+  if (rows <= 0) return hipSuccess;
+  hipLaunchKernelGGL(compact_kernel, dim3((rows + 3) / 4), dim3(256), 0, stream, kv_indices, kv_num, mask, rows,
+                     mask_stride, kv_len);
+  return hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------------
+// all_index_mask.  Reference: include/utils.cuh:73-93 (host loop + copy): every list is
+// 0,1,2,...,mask_stride-1 and every count is seq.  Here a store-only kernel.
+// ------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void all_index_kernel(int* __restrict__ kv_indices, int* __restrict__ kv_num,
+                                                        int rows, int mask_stride, int seq) {
+  const size_t vec_per_row = (size_t)mask_stride / 4;
+  const size_t nvec = vec_per_row * rows;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += (size_t)gridDim.x * blockDim.x) {
+    const int c = (int)(i % vec_per_row) * 4;
+    const i32x4 v = {c, c + 1, c + 2, c + 3};
+    reinterpret_cast<i32x4*>(kv_indices)[i] = v;
+  }
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < (size_t)rows; i += (size_t)gridDim.x * blockDim.x)
+    kv_num[i] = seq;
+}
+
+hipError_t run_all_index(int* kv_indices, int* kv_num, int rows, int mask_stride, int seq, hipStream_t stream) {
+  if (rows <= 0) return hipSuccess;
+  const size_t nvec = (size_t)mask_stride / 4 * rows;
+  size_t blocks = (nvec + 255) / 256;
+  if (blocks > 256 * 32) blocks = 256 * 32;
+  if (blocks == 0) blocks = 1;
+  hipLaunchKernelGGL(all_index_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, kv_indices, kv_num, rows,
+                     mask_stride, seq);
+  return hipGetLastError();
+}
+
+}  // namespace spattn

@@ -1,0 +1,119 @@
+/* C ABI of the gfx950 block-sparse attention library (libspattn_hip.so).
+ *
+ * Plain pointers and sizes only.  Every pointer is DEVICE memory (HIP), contiguous,
+ * 16-byte aligned.  q, k, v, o are bf16 [B,H,S,D] with D in {64,128}; index tensors are
+ * int32; statistics are fp32.  Nothing is allocated or kept between calls; the caller owns
+ * every buffer.  Kernels are enqueued asynchronously.
+ *
+ * Two groups of entry points:
+ *   1. the seven functions the reference's binding layer calls, with the reference's own
+ *      names and argument order (python/extension.cpp:4-49 declares them, python/cuda_attn.cu
+ *      defines them).  They run on the legacy default stream like the reference, return
+ *      nothing, and leave their status in spattn_last_status().
+ *   2. spattn_* variants that add what the reference lacks: a status return, a stream,
+ *      a runtime kv length, a softmax scale, a q-block size, an optional log-sum-exp
+ *      output, and KV-block index lists.
+ */
+#ifndef SPATTN_HIP_H_
+#define SPATTN_HIP_H_
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* status codes (0 = ok, >0 = hipError_t of the launch) */
+#define SPATTN_OK 0
+#define SPATTN_ERR_NULL -1       /* a required pointer is null */
+#define SPATTN_ERR_HEAD_DIM -2   /* D is not 64 or 128 */
+#define SPATTN_ERR_STRIDE -3     /* mask_stride is not a positive multiple of 128 */
+#define SPATTN_ERR_QBLK -4       /* q-block is not 64 or 128 */
+#define SPATTN_ERR_ALIGN -5      /* a pointer is not 16-byte aligned */
+#define SPATTN_ERR_SHAPE -6      /* a size is not positive / inconsistent */
+
+/* ---- group 1: the reference's binding surface ------------------------------------ */
+
+/* Dense attention o = softmax(q k^T / sqrt(D)) v.
+ * Replaces attn_fwd_wg_impl (python/extension.cpp:4-7, python/cuda_attn.cu:9-38). */
+void attn_fwd_wg_impl(void* o, void* q, void* k, void* v, int batch, int heads, int seq, int D);
+
+/* Gathered sparse attention: q-block I (128 rows) attends to the key tokens
+ * kv_indices[b][h][I][0 .. num_kv_indices[b][h][I]) ; kv_indices is [B,H,ceil(S/128),mask_stride].
+ * Replaces attn_sparse_fwd_wg_impl (python/extension.cpp:10-14, python/cuda_attn.cu:41-75). */
+void attn_sparse_fwd_wg_impl(void* o, void* q, void* k, void* v, int* kv_indices, int* num_kv_indices,
+                             int mask_stride, int batch, int heads, int seq, int D);
+
+/* Identity lists: kv_indices[b][h][I][s] = s for s < 128*ceil(seq/128), counts = seq.
+ * Replaces allindex_mask_impl (python/extension.cpp:17-20, python/cuda_attn.cu:78-94). */
+void allindex_mask_impl(int* kv_indices, int* num_kv_indices, int batch, int heads, int seqblocks, int seq);
+
+/* Dense attention that also writes the raw row max and the softmax denominator,
+ * both fp32 [B,H,1,128*ceil(S/128)]; pad rows get max 0 and denominator -inf.
+ * Replaces attn_maxq_denom_impl (python/extension.cpp:22-27, python/cuda_attn.cu:97-139). */
+void attn_maxq_denom_impl(void* d_o, float* d_o_max_q, float* d_o_norm, void* d_q, void* d_k, void* d_v, int batch,
+                          int heads, int seq, int D);
+
+/* Row max and denominator only.
+ * Replaces maxq_denom_impl (python/extension.cpp:29-33, python/cuda_attn.cu:142-180). */
+void maxq_denom_impl(float* d_o_max_q, float* d_o_norm, void* d_q, void* d_k, int batch, int heads, int seq, int D);
+
+/* Vote mask int32 [B,H,ceil(S/128),mask_stride]: entry (I,c) = number of 16-row groups of
+ * q-block I in which some row has softmax(r,c) > threshold.  The entry is stored (the
+ * reference adds into a caller-zeroed buffer; on a zeroed buffer the results agree).
+ * Replaces booleanmask_128_impl (python/extension.cpp:36-41, python/cuda_attn.cu:183-266). */
+void booleanmask_128_impl(int* d_booleanmask, float threshold, int mask_stride, float* d_o_max_q, float* d_o_norm,
+                          void* d_q, void* d_k, int batch, int heads, int seq, int D);
+
+/* Mask -> index lists: per row the keys c < seq with mask > 0 in ASCENDING order, then the
+ * caller's fill; counts are exact.  (The reference's order is whatever its atomics give.)
+ * Replaces booleanmask_to_indexmask_impl (python/extension.cpp:44-49, python/cuda_attn.cu:269-301). */
+void booleanmask_to_indexmask_impl(int* d_indexmask, int* d_num_indices, int* d_booleanmask, int batch, int heads,
+                                   int seq, int seqblocks, int mask_stride);
+
+/* ---- group 2: extended entry points ------------------------------------------------
+ * Common conventions: stream is a hipStream_t (NULL = legacy default stream);
+ * kv_len <= 0 means seq; scale <= 0 means 1/sqrt(D); lse may be NULL, else fp32 [B,H,S]
+ * natural-log log-sum-exp of the scaled scores over the attended keys.
+ * Each returns a status code and also records it for spattn_last_status(). */
+
+int spattn_full_attn(void* o, float* lse, const void* q, const void* k, const void* v, int batch, int heads, int seq,
+                     int D, int kv_len, float scale, void* stream);
+
+/* qblk in {64,128}: rows per q-block = rows sharing one list; kv_indices is
+ * [B,H,ceil(S/qblk),mask_stride]. */
+int spattn_sp_attn(void* o, float* lse, const void* q, const void* k, const void* v, const int* kv_indices,
+                   const int* num_kv_indices, int mask_stride, int qblk, int batch, int heads, int seq, int D,
+                   int kv_len, float scale, void* stream);
+
+/* KV-block lists: blk_indices int32 [B,H,ceil(S/qblk),max_blocks] holds 64-key block ids,
+ * blk_counts int32 [B,H,ceil(S/qblk)].  Block j stands for the tokens 64j .. 64j+63 (clipped
+ * to kv_len), so this is the token-list op restricted to aligned runs. */
+int spattn_sp_attn_blocks(void* o, float* lse, const void* q, const void* k, const void* v, const int* blk_indices,
+                          const int* blk_counts, int max_blocks, int qblk, int batch, int heads, int seq, int D,
+                          int kv_len, float scale, void* stream);
+
+int spattn_all_index_mask(int* kv_indices, int* num_kv_indices, int batch, int heads, int seqblocks, int seq,
+                          int mask_stride, void* stream);
+
+int spattn_fullattn_maxq_denom(void* o, float* max_q, float* denom, const void* q, const void* k, const void* v,
+                               int batch, int heads, int seq, int D, int kv_len, float scale, void* stream);
+
+int spattn_maxq_denom(float* max_q, float* denom, const void* q, const void* k, int batch, int heads, int seq, int D,
+                      int kv_len, float scale, void* stream);
+
+int spattn_booleanmask_128(int* booleanmask, float threshold, int mask_stride, const float* max_q, const float* denom,
+                           const void* q, const void* k, int batch, int heads, int seq, int D, int kv_len, float scale,
+                           void* stream);
+
+/* seq is the kv length (python/extension.cpp:326,338). */
+int spattn_booleanmask_to_indexmask(int* kv_indices, int* num_kv_indices, const int* booleanmask, int batch, int heads,
+                                    int seq, int seqblocks, int mask_stride, void* stream);
+
+/* Status of the most recent call on this host thread, and its text. */
+int spattn_last_status(void);
+const char* spattn_status_string(int status);
+int spattn_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SPATTN_HIP_H_ */

@@ -1,0 +1,101 @@
+"""GPU parity of the threshold pre-pass (statistics -> vote mask -> index lists)."""
+import numpy as np
+import pytest
+import torch
+
+from fgattn_tk_cuda_amd import capi, workloads as wl
+from oracle import spattn_oracle as orc
+from helpers import f32, to_dev
+
+pytestmark = pytest.mark.gpu
+
+BAND = 1e-2   # relative band around the threshold inside which a vote may flip
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("S,kv_len", [(512, 0), (1000, 0), (1000, 870)])
+def test_booleanmask_votes(dev, D, S, kv_len):
+    print("case booleanmask", D, S, kv_len, flush=True)
+    B, H = 1, 3
+    q, k, v = wl.clustered_qkv(B, H, S, D, seed=41, sigma=0.7)
+    qd, kd = to_dev(dev, q, k)
+    kv = kv_len or S
+    Sp = orc.padded_len(S)
+    SB = Sp // 128
+    mx = torch.empty((B, H, 1, Sp), device=dev)
+    dn = torch.empty((B, H, 1, Sp), device=dev)
+    capi.maxq_denom(mx, dn, qd, kd, kv_len=kv_len)
+    # threshold at the 70th percentile of the per-(q-block, key) peak probability
+    _, pmax0 = orc.booleanmask_128(f32(mx), f32(dn), f32(q), f32(k), 1.0, kv_len=kv)
+    thr = float(np.quantile(pmax0, 0.7))
+    mask = torch.full((B, H, SB, Sp), -7, dtype=torch.int32, device=dev)
+    capi.booleanmask_128(mask, mx, dn, qd, kd, thr, kv_len=kv_len)
+    got = mask.cpu().numpy()
+    votes, pmax = orc.booleanmask_128(f32(mx), f32(dn), f32(q), f32(k), thr, kv_len=kv)
+    assert got.min() >= 0 and got.max() <= 8
+    assert np.all(got[..., kv:] == 0)
+    near = np.abs(pmax - thr) <= BAND * thr
+    # outside the band the >0 masks must agree exactly
+    dis = ((got[..., :kv] > 0) != (votes[..., :kv] > 0)) & ~near
+    assert dis.sum() == 0, "%d mask mismatches outside the threshold band" % dis.sum()
+    # vote counts agree wherever no group sits in the band: check the bulk
+    frac_equal = (got[..., :kv] == votes[..., :kv]).mean()
+    assert frac_equal > 0.999, frac_equal
+    kept = (votes[..., :kv] > 0).mean()
+    assert 0.01 < kept < 0.9, kept
+
+
+@pytest.mark.parametrize("SB,ms,seq", [(3, 384, 300), (2, 2176, 2100), (5, 128, 128), (1, 4096, 1)])
+@pytest.mark.parametrize("density", [0.0, 0.08, 1.0])
+def test_compaction_bit_exact(dev, SB, ms, seq, density):
+    print("case compaction", SB, ms, seq, density, flush=True)
+    B, H = 2, 3
+    rng = np.random.default_rng(50)
+    mask = (rng.random((B, H, SB, ms)) < density).astype(np.int32) * rng.integers(1, 9, size=(B, H, SB, ms), dtype=np.int32)
+    md = torch.from_numpy(mask).to(dev)
+    kvi = torch.full((B, H, SB, ms), ms, dtype=torch.int32, device=dev)
+    kvn = torch.full((B, H, SB), -1, dtype=torch.int32, device=dev)
+    capi.booleanmask_to_indexmask(kvi, kvn, md, seq)
+    wi, wn = orc.booleanmask_to_indexmask(mask, seq)
+    assert np.array_equal(kvn.cpu().numpy(), wn)
+    assert np.array_equal(kvi.cpu().numpy(), wi)
+
+
+def test_all_index_mask(dev):
+    print("case all_index_mask", flush=True)
+    B, H, SB, S, ms = 2, 3, 5, 600, 640
+    kvi = torch.zeros((B, H, SB, ms), dtype=torch.int32, device=dev)
+    kvn = torch.zeros((B, H, SB), dtype=torch.int32, device=dev)
+    capi.all_index_mask(kvi, kvn, B, H, SB, S)
+    wi, wn = orc.all_index_mask(B, H, SB, S, ms)
+    assert np.array_equal(kvi.cpu().numpy(), wi) and np.array_equal(kvn.cpu().numpy(), wn)
+
+
+def test_threshold_pipeline_feeds_sparse_attention(dev):
+    """maxq_denom -> booleanmask_128 -> booleanmask_to_indexmask -> sp_attn on a padded length;
+    with a tiny threshold every key is kept and the result is dense attention."""
+    print("case pipeline", flush=True)
+    B, H, S, D = 1, 2, 1000, 64
+    q, k, v = wl.clustered_qkv(B, H, S, D, seed=61, sigma=0.7)
+    qd, kd, vd = to_dev(dev, q, k, v)
+    Sp = orc.padded_len(S)
+    SB = Sp // 128
+    mx = torch.empty((B, H, 1, Sp), device=dev)
+    dn = torch.empty((B, H, 1, Sp), device=dev)
+    capi.maxq_denom(mx, dn, qd, kd)
+    for thr, dense in ((1e-30, True), (0.05, False)):
+        mask = torch.zeros((B, H, SB, Sp), dtype=torch.int32, device=dev)
+        capi.booleanmask_128(mask, mx, dn, qd, kd, thr)
+        kvi = torch.full((B, H, SB, Sp), Sp, dtype=torch.int32, device=dev)
+        kvn = torch.zeros((B, H, SB), dtype=torch.int32, device=dev)
+        capi.booleanmask_to_indexmask(kvi, kvn, mask, S)
+        o = torch.full_like(qd, float("nan"))
+        capi.sp_attn(o, qd, kd, vd, kvi, kvn)
+        if dense:
+            assert np.all(kvn.cpu().numpy() == S)
+            want = f32(torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float()))
+        else:
+            want, _ = orc.sp_attn(f32(q), f32(k), f32(v), kvi.cpu().numpy(), kvn.cpu().numpy(), qblk=128)
+            assert 0 < kvn.float().mean().item() < S
+        from helpers import assert_close_o
+        assert_close_o(f32(o), want, "pipeline O (dense=%s)" % dense)
