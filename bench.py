@@ -1,0 +1,215 @@
+#!/usr/bin/env python3
+"""Benchmark of the gfx950 sparse-attention hot path on one MI355X.
+
+One "step" is one pass of gathered block-sparse attention over the headline workload
+(B=2, H=32, N=16384, d=128, 64x64 blocks, 26 of 256 key blocks per q-block row = 10 %
+density, seeded synthetic bf16 inputs already resident in HBM).  The JSON line reports
+kept-block TFLOP/s (4*64*64*128 flops per kept block), ms per step, the bf16-MFMA
+roofline fraction of the attention kernel, the HBM roofline fraction of the mask
+compaction stream (``mask_pass``), and a CPU baseline measured on this host's cores.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extras]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+from fgattn_tk_cuda_amd import capi, workloads as wl  # noqa: E402
+
+# MI355X published peaks
+PEAK_BF16_TFLOPS = 2500.0
+PEAK_HBM_GBPS = 8000.0
+
+
+def time_steps(fn, steps: int, warmup: int):
+    """Average milliseconds of fn() over `steps` launches, HIP events on the launch stream."""
+    stream = torch.cuda.current_stream()
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record(stream)
+    for _ in range(steps):
+        fn()
+    stop.record(stream)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    return start.elapsed_time(stop) / steps, wall_ms
+
+
+def bench_sparse(dev, steps, warmup, seed=0):
+    c = wl.CONFIGS["cfg3_sparse_16k"]
+    B, H, S, D, qblk, kvblk = c["B"], c["H"], c["S"], c["D"], c["qblk"], c["kvblk"]
+    nk = wl.ceil_div(S, kvblk)
+    count = int(round(c["density"] * nk))
+    q, k, v = (t.to(dev) for t in wl.randn_qkv(B, H, S, D, seed=seed))
+    bi, bc = (t.to(dev) for t in wl.uniform_block_lists(B, H, S, qblk, kvblk, count, seed=seed + 1))
+    o = torch.empty_like(q)
+    lse = torch.empty((B, H, S), dtype=torch.float32, device=dev)
+
+    def step():
+        capi.sp_attn_blocks(o, q, k, v, bi, bc, lse=lse, qblk=qblk)
+
+    ms, wall_ms = time_steps(step, steps, warmup)
+    kept = int(bc.sum().item())
+    flops = wl.kept_block_flops(kept, qblk, kvblk, D)
+    assert torch.isfinite(o.float()).all().item(), "non-finite attention output"
+    return dict(ms=ms, wall_ms=wall_ms, flops=flops, kept_blocks=kept, B=B, H=H, S=S, D=D, qblk=qblk, kvblk=kvblk,
+                count=count, tensors=(q, k, v, bi, bc, o))
+
+
+def bench_compaction(dev, steps, warmup, seed=0):
+    """booleanmask_to_indexmask at the padded threshold workload: B=1, H=24, N=32760 -> mask
+    [1,24,256,32768] int32 with ~8 % of the entries set."""
+    c = wl.CONFIGS["cfg4_threshold_padded"]
+    B, H, S = c["B"], c["H"], c["S"]
+    ms_ = 128 * wl.ceil_div(S, 128)
+    SB = ms_ // 128
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    mask = (torch.rand((B, H, SB, ms_), device=dev, generator=g) < c["keep"]).to(torch.int32)
+    kvi = torch.full((B, H, SB, ms_), ms_, dtype=torch.int32, device=dev)
+    kvn = torch.zeros((B, H, SB), dtype=torch.int32, device=dev)
+
+    def step():
+        capi.booleanmask_to_indexmask(kvi, kvn, mask, S)
+
+    ms, _ = time_steps(step, steps, warmup)
+    kept = int(kvn.sum().item())
+    nbytes = 4.0 * B * H * SB * ms_ + 4.0 * kept + 4.0 * B * H * SB
+    return dict(ms=ms, bytes=nbytes, kept=kept, shape=[B, H, SB, ms_])
+
+
+def bench_dense(dev, steps, warmup, seed=0):
+    c = wl.CONFIGS["cfg2_dense"]
+    B, H, S, D = c["B"], c["H"], c["S"], c["D"]
+    q, k, v = (t.to(dev) for t in wl.randn_qkv(B, H, S, D, seed=seed))
+    o = torch.empty_like(q)
+    ms, _ = time_steps(lambda: capi.full_attn(o, q, k, v), steps, warmup)
+    return dict(ms=ms, flops=4.0 * B * H * S * S * D)
+
+
+def bench_sweeps(dev, steps, warmup, seed=0, heads=None):
+    """The two QK^T sweeps of the pre-pass (maxq_denom, booleanmask_128) at B=1,H=24,N=32760,d=64."""
+    c = wl.CONFIGS["cfg4_threshold_padded"]
+    B, H, S, D = c["B"], heads or c["H"], c["S"], c["D"]
+    q, k, _ = (t.to(dev) for t in wl.clustered_qkv(B, H, S, D, seed=seed))
+    Sp = 128 * wl.ceil_div(S, 128)
+    mx = torch.empty((B, H, 1, Sp), device=dev)
+    dn = torch.empty((B, H, 1, Sp), device=dev)
+    mask = torch.zeros((B, H, Sp // 128, Sp), dtype=torch.int32, device=dev)
+    ms1, _ = time_steps(lambda: capi.maxq_denom(mx, dn, q, k), steps, warmup)
+    ms2, _ = time_steps(lambda: capi.booleanmask_128(mask, mx, dn, q, k, 1e-3), steps, warmup)
+    flops = 2.0 * B * H * float(Sp) * Sp * D
+    return dict(ms_maxq_denom=ms1, ms_booleanmask=ms2, flops=flops, mask_bytes=4.0 * mask.numel())
+
+
+def cpu_baseline(res, budget_s=20.0):
+    """Dense-masked PyTorch attention on the host cores over a bounded sample of the
+    headline workload: whole q-blocks of head (0,0), as many as fit the time budget."""
+    from oracle import cpu_masked_attention as cma
+
+    q, k, v, bi, bc, _ = res["tensors"]
+    S, D, qblk, kvblk = res["S"], res["D"], res["qblk"], res["kvblk"]
+    qh, kh, vh = (t[0, 0].float().cpu() for t in (q, k, v))
+    bih, bch = bi[0, 0].cpu(), bc[0, 0].cpu()
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    chunk = 2048
+    done_rows, kept, t_used = 0, 0, 0.0
+    while done_rows < S and t_used < budget_s:
+        r0, r1 = done_rows, min(S, done_rows + chunk)
+        t0 = time.perf_counter()
+        cma.masked_attention_rows(qh, kh, vh, bih, bch, r0, r1, qblk, kvblk)
+        t_used += time.perf_counter() - t0
+        kept += int(bch[r0 // qblk: wl.ceil_div(r1, qblk)].sum())
+        done_rows = r1
+    flops = wl.kept_block_flops(kept, qblk, kvblk, D)
+    return {
+        "value": flops / t_used / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+        "sample": "dense-masked fp32 torch attention (QK^T, -inf outside kept blocks, softmax, PV) on %d of %d query "
+                  "rows of head (0,0), %.1f s; kept-block flops of those rows / time" % (done_rows, S, t_used),
+        "seconds": t_used,
+    }
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-extras", action="store_true", help="only the headline kernel")
+    ap.add_argument("--only", default="", help="run one leg only: sparse|compact|dense|sweeps (no JSON contract)")
+    args = ap.parse_args(argv)
+    if args.gpus != 1:
+        print("bench.py: this library is single-GPU; run with --gpus 1 (got %d)" % args.gpus, file=sys.stderr)
+        return 2
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 2
+    capi.load()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    if args.only:
+        fn = {"sparse": bench_sparse, "compact": bench_compaction, "dense": bench_dense, "sweeps": bench_sweeps}[args.only]
+        r = fn(dev, args.steps, args.warmup)
+        r.pop("tensors", None)
+        print(json.dumps(r))
+        return 0
+
+    res = bench_sparse(dev, args.steps, args.warmup)
+    tflops = res["flops"] / (res["ms"] * 1e-3) / 1e12
+    out = {
+        "metric": "kept-block TFLOP/s, gathered block-sparse attention N=16K d=128 10% density",
+        "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": res["ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "cfg3: sp_attn over KV-block lists, B=2 H=32 N=16384 d=128, q-block 64, kv-block 64, "
+                               "26 of 256 key blocks per row incl. diagonal, bf16 O + fp32 lse",
+                   "kept_blocks": res["kept_blocks"], "flops_per_step": res["flops"]},
+        "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": None,
+                     "kernel": "attn_fwd_kernel<128,64,KV_BLOCKS>"},
+    }
+    if not args.no_extras:
+        cp = bench_compaction(dev, args.steps, args.warmup)
+        gbps = cp["bytes"] / (cp["ms"] * 1e-3) / 1e9
+        out["mask_pass"] = {"kernel": "compact_kernel (booleanmask_to_indexmask)", "workload": "cfg4 mask %s int32, %.1f%% kept"
+                            % (cp["shape"], 100.0 * cp["kept"] / np.prod(cp["shape"])), "ms": cp["ms"],
+                            "roofline": {"bound": "hbm", "achieved": gbps, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                                         "frac": gbps / PEAK_HBM_GBPS, "traffic": None}}
+        dn = bench_dense(dev, args.steps, args.warmup)
+        out["dense_full_attn"] = {"workload": "cfg2: B=4 H=16 N=4096 d=64", "ms": dn["ms"],
+                                  "tflops": dn["flops"] / (dn["ms"] * 1e-3) / 1e12,
+                                  "mfma_frac": dn["flops"] / (dn["ms"] * 1e-3) / 1e12 / PEAK_BF16_TFLOPS}
+        sw = bench_sweeps(dev, max(2, args.steps // 5), 1)
+        out["prepass_sweeps"] = {
+            "workload": "cfg4: B=1 H=24 N=32760 d=64",
+            "maxq_denom_ms": sw["ms_maxq_denom"], "maxq_denom_tflops": sw["flops"] / sw["ms_maxq_denom"] / 1e9,
+            "booleanmask_128_ms": sw["ms_booleanmask"], "booleanmask_128_tflops": sw["flops"] / sw["ms_booleanmask"] / 1e9,
+            "booleanmask_128_write_gbps": sw["mask_bytes"] / sw["ms_booleanmask"] / 1e6}
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(res)
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
