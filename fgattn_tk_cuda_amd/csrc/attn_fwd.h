@@ -7,12 +7,12 @@
 //   include/maxq_denom_attn.cuh:196-252                 (dense attention + row statistics),
 //   include/maxq_denom.cuh:169-206                      (row statistics only):
 // running raw row max m, p = exp2((s - m) * log2e * scale), fp32 denominator, P rounded
-// to bf16 before PV, O / l at the end.  Keys that are out of range (list position >= n,
+// to bf16 before PV, O / l at the end.  Keys that do not exist (list position >= n,
 // token id >= kv_len, row >= kv_len) are masked on every tile, a superset of the
 // reference's "NaN row -> -inf on the last tile" (include/asyncloadutils.cuh:124-142,
 // include/pad_utils.cuh:54-75).
 //
-// Layout.  A workgroup is 4 waves (256 lanes) and owns one q-block of QBLK rows.
+// Work split.  A workgroup is 4 waves (256 lanes) and owns one q-block of QBLK rows.
 // Scores are produced transposed, S^T = K Q^T, so that in the 32x32 MFMA accumulator a
 // lane holds ONE query row (n = lane & 31) and 16 keys: every softmax statistic is a
 // per-lane scalar and only lanes l and l^32 ever exchange data.  O is accumulated
@@ -20,30 +20,57 @@
 //   QBLK = 128: wave w owns query rows 32w..32w+31 and all 64 keys of a tile.
 //   QBLK =  64: wave w owns query rows 32(w&1).. and keys 32(w>>1).. of a tile; the two
 //               key halves are merged through LDS at the end.
-// LDS per stage: K tile [64][D] bf16 (16-byte chunks XOR-swizzled by row), V^T tile
-// [D][64] bf16 (keys permuted so that the PV operand is one 16-byte read), 64 bias
-// floats.  Two stages, one barrier per tile; the next tile's rows travel
-// HBM -> registers while the current tile is multiplied.
+//
+// Data movement.  K and V tiles (64 rows x D bf16, row-major as in HBM) go HBM -> LDS with
+// global_load_lds_dwordx4: no staging registers, no LDS stores.  Each lane picks which
+// 16-byte chunk of its row it fetches so that the tile lands XOR-swizzled (K: chunk ^
+// row; V: chunk ^ 2*(row&7)).  K is read back as the MFMA A operand with ds_read_b128; the
+// V^T operand comes from ds_read_b64_tr_b16, which hands lane j of a 16-lane group the
+// j-th 16-bit column of the 4 rows the group addressed.  Tiles live in a ring of kSlots
+// slots consumed in the order K0 V0 K1 V1 ...; every phase is
+//     wait own loads of this phase -> barrier -> issue the load kSlots-1 phases ahead
+//     into the slot the barrier just freed -> multiply,
+// so kSlots-1 tiles are always in flight per workgroup.
 #pragma once
 #include "common.h"
 
 namespace spattn {
 
-template <int D, bool HAS_V>
-struct AttnSmem {
-  static constexpr int kKBytes = 64 * D * 2;
-  static constexpr int kVBytes = HAS_V ? D * 64 * 2 : 0;
-  static constexpr int kBiasBytes = 64 * 4;
-  static constexpr int kStage = kKBytes + kVBytes + kBiasBytes;
-  // The key-split merge needs 2 waves * (D/2 + 2) * 64 floats; it reuses the stages.
-  static constexpr int kMerge = 2 * (D / 2 + 2) * 64 * 4;
-  static constexpr int kTotal = (2 * kStage > kMerge) ? 2 * kStage : kMerge;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+#define SPATTN_LDS __attribute__((address_space(3)))
+
+template <int D, int MODE, bool HAS_V>
+struct AttnCfg {
+  static constexpr int kTileBytes = 64 * D * 2;
+  // D=128: 5 x 16 KB = 80 KB, two workgroups fill the 160 KB of a CU exactly.
+  static constexpr int kSlots = (D == 128) ? (MODE == KV_TOKENS ? 4 : 5) : 8;
+  static constexpr int kLead = kSlots - 1;                 // phases between issue and use
+  static constexpr int kBiasRing = 4;                       // tiles of key-validity bias (token lists)
+  static constexpr int kBiasBytes = (MODE == KV_TOKENS) ? kBiasRing * 64 * 4 : 0;
+  static constexpr int kRing = kSlots * kTileBytes;
+  static constexpr int kMerge = 2 * (D / 2 + 2) * 64 * 4;   // key-split merge, overlays the ring
+  static constexpr int kTotal = ((kRing > kMerge) ? kRing : kMerge) + kBiasBytes;
+  static constexpr int kRowsPerLoad = 1024 / (D * 2);       // rows one wave-wide 1 KB load covers
+  static constexpr int kLoadsPerTile = kTileBytes / 1024 / 4;   // per wave
 };
+
+// One wave-wide HBM -> LDS copy: lane l's 16 bytes land at lds_base + 16 l.
+__device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_base) {
+  // Written as asm on purpose: the compiler does not count this load in its own vmcnt
+  // bookkeeping (with the builtin it drains every outstanding load before each LDS read),
+  // so the waits below are placed by hand.
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(gptr) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
 
 template <int D, int QBLK, int MODE, bool HAS_V, bool STATS>
 __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   static_assert(D == 64 || D == 128, "head dim");
   static_assert(QBLK == 64 || QBLK == 128, "q-block");
+  using Cfg = AttnCfg<D, MODE, HAS_V>;
   constexpr int NQW = QBLK / 32;     // waves along the query rows
   constexpr int KSPLIT = 4 / NQW;    // waves along the keys of a tile
   constexpr int KW = 64 / KSPLIT;    // keys of a tile per wave
@@ -51,15 +78,21 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   constexpr int NT = D / 16;         // k-steps of the QK^T product
   constexpr int NDB = D / 32;        // 32-wide blocks of the head dim
   constexpr int NKS = KW / 16;       // k-steps of the PV product
-  constexpr int CPR = D / 8;         // 16-byte chunks per K row
-  using Smem = AttnSmem<D, HAS_V>;
+  constexpr int CPR = D / 8;         // 16-byte chunks per row
+  constexpr int ROWB = D * 2;        // bytes per row
+  constexpr int SLOTS = Cfg::kSlots;
+  constexpr int LEAD = Cfg::kLead;
+  constexpr int LPT = Cfg::kLoadsPerTile;
+  constexpr int RPL = Cfg::kRowsPerLoad;
+  constexpr int PPT = HAS_V ? 2 : 1;   // phases per tile
   constexpr float kNegInf = -__builtin_huge_valf();
 
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  const uint32_t smem_base = (uint32_t)(uintptr_t)(SPATTN_LDS unsigned char*)smem;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ln = lane & 31;
   const int g = lane >> 5;
   const int qsub = wave % NQW;
@@ -72,111 +105,127 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
 
   const size_t head_off = (size_t)bh * p.S * D;
   const uint16_t* __restrict__ qh = p.q + head_off;
-  const uint16_t* __restrict__ kh = p.k + head_off;
-  const uint16_t* __restrict__ vh = HAS_V ? p.v + head_off : nullptr;
+  const unsigned char* __restrict__ kh = reinterpret_cast<const unsigned char*>(p.k + head_off);
+  const unsigned char* __restrict__ vh = HAS_V ? reinterpret_cast<const unsigned char*>(p.v + head_off) : nullptr;
 
   // ---- tile list of this q-block -------------------------------------------------
-  const int* __restrict__ lst = nullptr;
+  // The lists are read through the constant address space: with a wave-uniform address
+  // that makes them scalar loads, which stay out of the vector-memory counter that the
+  // tile pipeline waits on.
+  typedef const __attribute__((address_space(4))) int* cint_p;
+  cint_p lst = nullptr;
   int n = 0, ntiles = 0;
   if constexpr (MODE == KV_DENSE) {
     ntiles = (p.kv_len + 63) >> 6;
   } else {
     const size_t lrow = (size_t)bh * p.nqblk + qb;
-    lst = p.idx + lrow * p.idx_stride;
-    n = p.cnt[lrow];
+    lst = (cint_p)(p.idx + lrow * p.idx_stride);
+    n = ((cint_p)p.cnt)[lrow];
     n = n < 0 ? 0 : (n > p.idx_stride ? p.idx_stride : n);
     ntiles = (MODE == KV_TOKENS) ? ((n + 63) >> 6) : n;
   }
+  const int nphase = ntiles * PPT;
+  const int last_row = p.kv_len - 1;
 
-  // ---- loader role of this thread ------------------------------------------------
-  constexpr bool SPLIT_ROLES = (D == 64);
-  const int tt = SPLIT_ROLES ? (tid & 127) : tid;
-  const bool k_loader = SPLIT_ROLES ? (tid < 128) : true;
-  const bool v_loader = HAS_V && (SPLIT_ROLES ? (tid >= 128) : true);
-  const int ld_c = tt % CPR;         // 16-byte chunk of the row
-  const int ld_a = tt / CPR;         // rows 4*ld_a .. 4*ld_a+3 of the tile
-  // V^T column of key 4*ld_a: the two low bits of ld_a swapped (see the PV operand below).
-  const int ld_ap = (ld_a & ~3) | ((ld_a & 1) << 1) | ((ld_a >> 1) & 1);
-
-  // Row sources of one tile for this thread.
-  struct Rows {
-    int row[4];
-    bool ok[4];
-  };
-  auto raw_index = [&](int it) -> i32x4 {
-    i32x4 r = {0, 0, 0, 0};
-    if (it < ntiles) {
-      if constexpr (MODE == KV_TOKENS) r = *reinterpret_cast<const i32x4*>(lst + it * 64 + 4 * ld_a);
-      if constexpr (MODE == KV_BLOCKS) r[0] = lst[it];
-    }
-    return r;
-  };
-  auto resolve = [&](int it, i32x4 raw) -> Rows {
-    Rows r;
+  // ---- loader role: load i of a tile covers rows RPL*(4i + wave) .. +RPL-1 ----------
+  const int ld_sub = lane / CPR;       // row within the load
+  const int ld_slot = lane % CPR;      // 16-byte position within the row in LDS
+  int ld_row[LPT];
+  int ld_koff[LPT], ld_voff[LPT];      // byte offset of this lane's chunk within its row
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      if constexpr (MODE == KV_DENSE) {
-        r.row[i] = it * 64 + 4 * ld_a + i;
-        r.ok[i] = r.row[i] < p.kv_len;
-      } else if constexpr (MODE == KV_BLOCKS) {
-        const int blk = raw[0];
-        r.row[i] = blk * 64 + 4 * ld_a + i;
-        r.ok[i] = blk >= 0 && blk <= (p.kv_len >> 6) && r.row[i] < p.kv_len;
-      } else {
-        r.row[i] = raw[i];
-        r.ok[i] = (it * 64 + 4 * ld_a + i) < n && (unsigned)raw[i] < (unsigned)p.kv_len;
-      }
+  for (int i = 0; i < LPT; ++i) {
+    const int r = RPL * (4 * i + wave) + ld_sub;
+    ld_row[i] = r;
+    ld_koff[i] = (ld_slot ^ (r & (CPR - 1))) << 4;
+    ld_voff[i] = (ld_slot ^ ((r & (D == 128 ? 7 : 3)) << 1)) << 4;
+  }
+
+  // First key row of tile t (dense / block lists); kv_len marks "no such block".
+  auto tile_row0 = [&](int t) -> int {
+    if constexpr (MODE == KV_DENSE) return t * 64;
+    if constexpr (MODE == KV_BLOCKS) {
+      const int blk = lst[t];
+      return (blk >= 0 && blk <= (last_row >> 6)) ? blk * 64 : p.kv_len;
     }
-    return r;
+    return 0;
   };
 
-  u32x4 kr[4], vr[4];
-  float bias_r[4];
-  auto issue_loads = [&](const Rows& r) {
+  // Token lists: the RPL token ids behind one load are wave-uniform, so they are fetched
+  // as scalars (tok_raw) one tile ahead and turned into this lane's row (tok_row) just
+  // before the K and V loads of that tile are issued.
+  int tok_raw[MODE == KV_TOKENS ? LPT : 1][MODE == KV_TOKENS ? RPL : 1];
+  int tok_row[MODE == KV_TOKENS ? LPT : 1];
+  bool tok_ok[MODE == KV_TOKENS ? LPT : 1];
+  auto tok_fetch = [&](int t) {
+    if constexpr (MODE == KV_TOKENS) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const u32x4 z = {0, 0, 0, 0};
-      kr[i] = z;
-      vr[i] = z;
-      bias_r[i] = r.ok[i] ? 0.f : kNegInf;
-      if (r.ok[i]) {
-        const size_t off = (size_t)r.row[i] * D + 8 * ld_c;
-        if (k_loader) kr[i] = *reinterpret_cast<const u32x4*>(kh + off);
-        if (v_loader) vr[i] = *reinterpret_cast<const u32x4*>(vh + off);
-      }
+      for (int i = 0; i < LPT; ++i)
+#pragma unroll
+        for (int s = 0; s < RPL; ++s) tok_raw[i][s] = (t < ntiles) ? lst[t * 64 + RPL * (4 * i + wave) + s] : 0;
     }
   };
-  auto store_tile = [&](int stage) {
-    unsigned char* kb = smem + stage * Smem::kStage;
-    if (k_loader) {
+  auto tok_resolve = [&](int t) {
+    if constexpr (MODE == KV_TOKENS) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int r = 4 * ld_a + i;
-        *reinterpret_cast<u32x4*>(kb + r * (D * 2) + ((ld_c ^ (r & (CPR - 1))) << 4)) = kr[i];
-      }
-      if (MODE == KV_TOKENS && ld_c == 0) {
-        float* bias = reinterpret_cast<float*>(kb + Smem::kKBytes + Smem::kVBytes);
-        *reinterpret_cast<float4*>(bias + 4 * ld_a) = make_float4(bias_r[0], bias_r[1], bias_r[2], bias_r[3]);
-      }
-    }
-    if constexpr (HAS_V) {
-      if (v_loader) {
-        unsigned char* vb = kb + Smem::kKBytes;
-        // Transpose the 4 keys x 8 dims held in registers into 8 dims x 4 keys.
+      for (int i = 0; i < LPT; ++i) {
+        int tok = 0;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
-#pragma unroll
-          for (int hl = 0; hl < 2; ++hl) {
-            const uint32_t sel = hl ? 0x07060302u : 0x05040100u;
-            u32x2 out;
-            out[0] = __builtin_amdgcn_perm(vr[1][w], vr[0][w], sel);
-            out[1] = __builtin_amdgcn_perm(vr[3][w], vr[2][w], sel);
-            const int d = 8 * ld_c + 2 * w + hl;
-            const int unit = (ld_ap >> 1) ^ ((d ^ (d >> 3)) & 7);
-            *reinterpret_cast<u32x2*>(vb + d * 128 + (unit << 4) + ((ld_ap & 1) << 3)) = out;
-          }
+        for (int s = 0; s < RPL; ++s) {
+          int v = tok_raw[i][s];
+          asm volatile("" : "+s"(v));   // keep it a scalar: no per-lane reload of the list
+          tok = (ld_sub == s) ? v : tok;
         }
+        tok_ok[i] = (t * 64 + ld_row[i]) < n && (unsigned)tok <= (unsigned)last_row;
+        tok_row[i] = tok_ok[i] ? tok : 0;
       }
+    }
+  };
+
+  // Issue the loads of phase jj (tile jj / PPT; K if even or no V, else V).  Phases are
+  // issued strictly in order, which the token-id prefetch relies on.
+  auto issue = [&](int jj) {
+    if (jj >= nphase) return;
+    const int t = HAS_V ? (jj >> 1) : jj;
+    const bool is_v = HAS_V && (jj & 1);
+    const uint32_t slot_base = smem_base + (uint32_t)(jj % SLOTS) * Cfg::kTileBytes;
+    const unsigned char* src = is_v ? vh : kh;
+    if constexpr (MODE == KV_TOKENS) {
+      float* bias = reinterpret_cast<float*>(smem + Cfg::kTotal - Cfg::kBiasBytes) + (t % Cfg::kBiasRing) * 64;
+#pragma unroll
+      for (int i = 0; i < LPT; ++i) {
+        dma16(src + (size_t)tok_row[i] * ROWB + (is_v ? ld_voff[i] : ld_koff[i]), slot_base + (4 * i + wave) * 1024);
+        if (!is_v && ld_slot == 0) bias[ld_row[i]] = tok_ok[i] ? 0.f : kNegInf;
+      }
+      if (is_v || !HAS_V) {
+        tok_resolve(t + 1);
+        tok_fetch(t + 2);
+      }
+    } else {
+      const int r0 = tile_row0(t);
+#pragma unroll
+      for (int i = 0; i < LPT; ++i) {
+        int row = r0 + ld_row[i];
+        row = row > last_row ? last_row : row;
+        dma16(src + (size_t)row * ROWB + (is_v ? ld_voff[i] : ld_koff[i]), slot_base + (4 * i + wave) * 1024);
+      }
+    }
+  };
+
+  // Wait until this wave's loads of phase j have landed: everything issued after them
+  // (up to LEAD-1 phases) may stay in flight.
+  auto wait_phase = [&](int j) {
+    const int later = nphase - 1 - j;   // phases issued after j
+    if (later >= LEAD - 1) {
+      wait_vmcnt<(LEAD - 1) * LPT>();
+    } else {
+      // tail: fewer loads behind this one
+      if constexpr (LEAD - 1 > 6) if (later == 6) { wait_vmcnt<6 * LPT>(); return; }
+      if constexpr (LEAD - 1 > 5) if (later == 5) { wait_vmcnt<5 * LPT>(); return; }
+      if constexpr (LEAD - 1 > 4) if (later == 4) { wait_vmcnt<4 * LPT>(); return; }
+      if constexpr (LEAD - 1 > 3) if (later == 3) { wait_vmcnt<3 * LPT>(); return; }
+      if constexpr (LEAD - 1 > 2) if (later == 2) { wait_vmcnt<2 * LPT>(); return; }
+      if constexpr (LEAD - 1 > 1) if (later == 1) { wait_vmcnt<1 * LPT>(); return; }
+      wait_vmcnt<0>();
     }
   };
 
@@ -184,6 +233,23 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   const int q0 = qb * QBLK + qsub * 32;
   const int qrow = q0 + ln;
   const bool qrow_ok = qrow < p.S;
+
+  u32x4 qf[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const u32x4 z = {0, 0, 0, 0};
+    qf[t] = qrow_ok ? *reinterpret_cast<const u32x4*>(qh + (size_t)qrow * D + 16 * t + 8 * g) : z;
+  }
+  // The Q loads must have retired before the first counted wait; they are the only
+  // compiler-visible vector loads of the kernel.
+#pragma unroll
+  for (int t = 0; t < NT; ++t) asm volatile("" ::"v"(qf[t]));
+
+  tok_fetch(0);
+  tok_resolve(0);
+  tok_fetch(1);
+#pragma unroll
+  for (int jj = 0; jj < LEAD; ++jj) issue(jj);
 
   float m_run = kNegInf;   // running raw row max
   float l_run = 0.f;       // running denominator, this lane's keys only
@@ -193,48 +259,23 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
 
-  u32x4 qf[NT];
-#pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    const u32x4 z = {0, 0, 0, 0};
-    qf[t] = qrow_ok ? *reinterpret_cast<const u32x4*>(qh + (size_t)qrow * D + 16 * t + 8 * g) : z;
-  }
+  u32x4 pb[HAS_V ? NKS : 1];
 
-  if (ntiles > 0) {
-    i32x4 raw_cur = raw_index(0);
-    i32x4 raw_nxt = raw_index(1);
-    int tile_row0 = 0;   // dense/block: first key row of the current tile
-    {
-      Rows r0 = resolve(0, raw_cur);
-      issue_loads(r0);
-      store_tile(0);
-    }
+  for (int it = 0; it < ntiles; ++it) {
+    // ================= K phase: S^T = K Q^T, online softmax =================
+    const int jk = it * PPT;
+    wait_phase(jk);
     __syncthreads();
-
-    for (int it = 0; it < ntiles; ++it) {
-      const int cur = it & 1;
-      if constexpr (MODE == KV_DENSE) tile_row0 = it * 64;
-      if constexpr (MODE == KV_BLOCKS) {
-        const int blk = raw_cur[0];
-        tile_row0 = (blk >= 0 && blk <= (p.kv_len >> 6)) ? blk * 64 : p.kv_len;
-      }
-      const bool has_next = (it + 1) < ntiles;
-      if (has_next) {
-        Rows rn = resolve(it + 1, raw_nxt);
-        issue_loads(rn);
-      }
-      raw_cur = raw_nxt;
-      raw_nxt = raw_index(it + 2);
-
-      // ---- S^T = K Q^T for this wave's keys ----
-      const unsigned char* kb = smem + cur * Smem::kStage;
+    issue(jk + LEAD);
+    {
+      const unsigned char* kb = smem + (jk % SLOTS) * Cfg::kTileBytes;
       f32x16 s[NMB];
 #pragma unroll
       for (int mb = 0; mb < NMB; ++mb) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[mb][r] = 0.f;
         const int krow = ksub * KW + mb * 32 + ln;
-        const unsigned char* krp = kb + krow * (D * 2);
+        const unsigned char* krp = kb + krow * ROWB;
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
           const u32x4 a = *reinterpret_cast<const u32x4*>(krp + (((2 * t + g) ^ (krow & (CPR - 1))) << 4));
@@ -245,7 +286,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
       // ---- mask keys that do not exist ----
       // Accumulator register 4j+i of block mb is key ksub*KW + 32mb + 8j + 4g + i of the tile.
       if constexpr (MODE == KV_TOKENS) {
-        const float* bias = reinterpret_cast<const float*>(kb + Smem::kKBytes + Smem::kVBytes);
+        const float* bias = reinterpret_cast<const float*>(smem + Cfg::kTotal - Cfg::kBiasBytes) + (it % Cfg::kBiasRing) * 64;
 #pragma unroll
         for (int mb = 0; mb < NMB; ++mb)
 #pragma unroll
@@ -257,12 +298,13 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
             s[mb][4 * j + 3] += bv.w;
           }
       } else {
-        if (tile_row0 + 64 > p.kv_len) {
+        const int r0 = tile_row0(it);
+        if (r0 + 64 > p.kv_len) {
 #pragma unroll
           for (int mb = 0; mb < NMB; ++mb)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-              const int key = tile_row0 + ksub * KW + 32 * mb + 8 * (r >> 2) + 4 * g + (r & 3);
+              const int key = r0 + ksub * KW + 32 * mb + 8 * (r >> 2) + 4 * g + (r & 3);
               if (key >= p.kv_len) s[mb][r] = kNegInf;
             }
         }
@@ -297,9 +339,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
         }
-        // P^T operand: registers 8h..8h+7 of block mb are the 8 keys this lane feeds to
-        // k-step 2mb+h; the V^T tile stores those keys at columns 16(2mb+h) + 8g + 0..7.
-        u32x4 pb[NKS];
+        // P^T operand of k-step ks = 2mb+h: registers 8h..8h+7 of block mb, i.e. keys
+        // 32mb + 16h + {4g..4g+3} and 32mb + 16h + 8 + {4g..4g+3}.
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks) {
           const int mb = ks >> 1, h8 = (ks & 1) * 8;
@@ -308,25 +349,45 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
           pb[ks][2] = pack_bf16(s[mb][h8 + 4], s[mb][h8 + 5]);
           pb[ks][3] = pack_bf16(s[mb][h8 + 6], s[mb][h8 + 7]);
         }
-        const unsigned char* vb = kb + Smem::kKBytes;
+      }
+    }
+
+    // ================= V phase: O^T += V^T P^T =================
+    if constexpr (HAS_V) {
+      const int jv = jk + 1;
+      wait_phase(jv);
+      __syncthreads();
+      issue(jv + LEAD);
+      const unsigned char* vb = smem + (jv % SLOTS) * Cfg::kTileBytes;
+      // Transposing read: in each 16-lane group, lane i addresses 4 dims of key (i>>2);
+      // lane j receives dim j of those 4 keys.
+      const int i16 = lane & 15;
+      const int dhalf = (lane >> 4) & 1;
+      const int rsub = i16 >> 2;                               // key within the group of 4
+      const int cb = 2 * dhalf + ((i16 & 3) >> 1);             // 16-byte chunk within the 32-dim block
+      const int bofs = (i16 & 1) << 3;                         // 8-byte half of the chunk
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) {
+        const int r1 = ksub * KW + 16 * ks + 4 * g + rsub;     // keys of A columns 8g+0..3
+        const int r2 = r1 + 8;                                 // keys of A columns 8g+4..7
+        const int sw1 = (r1 & (D == 128 ? 7 : 3)) << 1;
+        const int sw2 = (r2 & (D == 128 ? 7 : 3)) << 1;
+        const unsigned char* p1 = vb + r1 * ROWB + bofs;
+        const unsigned char* p2 = vb + r2 * ROWB + bofs;
 #pragma unroll
         for (int db = 0; db < NDB; ++db) {
-          const int d = 32 * db + ln;
-          const unsigned char* vrp = vb + d * 128;
-          const int hsw = (d ^ (d >> 3)) & 7;
-#pragma unroll
-          for (int ks = 0; ks < NKS; ++ks) {
-            const int unit = (ksub * KW + 16 * ks + 8 * g) >> 3;
-            const u32x4 a = *reinterpret_cast<const u32x4*>(vrp + ((unit ^ hsw) << 4));
-            oacc[db] = mfma32(a, pb[ks], oacc[db]);
-          }
+          const int c = 4 * db + cb;
+          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((SPATTN_LDS s16x4*)(p1 + ((c ^ sw1) << 4)));
+          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((SPATTN_LDS s16x4*)(p2 + ((c ^ sw2) << 4)));
+          const u32x2 lo2 = __builtin_bit_cast(u32x2, lo);
+          const u32x2 hi2 = __builtin_bit_cast(u32x2, hi);
+          const u32x4 a = {lo2[0], lo2[1], hi2[0], hi2[1]};
+          oacc[db] = mfma32(a, pb[ks], oacc[db]);
         }
       }
-
-      if (has_next) store_tile(cur ^ 1);
-      __syncthreads();
     }
   }
+  __syncthreads();   // every wave is done with the ring
 
   // ---- combine the two 32-lane halves, then the two key halves -------------------
   float l_tot = l_run + xor32(l_run);
@@ -395,17 +456,17 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
 // Host launcher; returns hipError_t of the launch.
 template <int D, int QBLK, int MODE, bool HAS_V, bool STATS>
 inline hipError_t launch_attn_fwd(const AttnParams& p, hipStream_t stream) {
-  using Smem = AttnSmem<D, HAS_V>;
+  using Cfg = AttnCfg<D, MODE, HAS_V>;
   auto kern = attn_fwd_kernel<D, QBLK, MODE, HAS_V, STATS>;
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, Smem::kTotal);
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kTotal);
     if (e != hipSuccess) return e;
     attr_set = true;
   }
   const int total = p.nqblk * p.H * p.B;
   if (total <= 0) return hipSuccess;
-  hipLaunchKernelGGL(kern, dim3(total), dim3(256), Smem::kTotal, stream, p);
+  hipLaunchKernelGGL(kern, dim3(total), dim3(256), Cfg::kTotal, stream, p);
   return hipGetLastError();
 }
 
