@@ -48,7 +48,7 @@ struct AttnCfg {
   static constexpr int kBiasRing = 4;                       // tiles of key-validity bias (token lists)
   static constexpr int kBiasBytes = (MODE == KV_TOKENS) ? kBiasRing * 64 * 4 : 0;
   static constexpr int kRing = kSlots * kTileBytes;
-  static constexpr int kMerge = 2 * (D / 2 + 2) * 64 * 4;   // key-split merge, overlays the ring
+  static constexpr int kMerge = 2 * (D / 2 + 3) * 64 * 4;   // key-split merge, overlays the ring
   static constexpr int kTotal = ((kRing > kMerge) ? kRing : kMerge) + kBiasBytes;
   static constexpr int kRowsPerLoad = 1024 / (D * 2);       // rows one wave-wide 1 KB load covers
   static constexpr int kLoadsPerTile = kTileBytes / 1024 / 4;   // per wave
@@ -60,6 +60,10 @@ __device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_base) {
   // bookkeeping (with the builtin it drains every outstanding load before each LDS read),
   // so the waits below are placed by hand.
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(gptr) : "memory");
+}
+// Same with a wave-uniform base pointer and a 32-bit per-lane byte offset.
+__device__ __forceinline__ void dma16(const void* sbase, uint32_t voff, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(voff), "s"(sbase) : "memory");
 }
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
@@ -132,12 +136,15 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   const int ld_slot = lane % CPR;      // 16-byte position within the row in LDS
   int ld_row[LPT];
   int ld_koff[LPT], ld_voff[LPT];      // byte offset of this lane's chunk within its row
+  uint32_t ld_kgo[LPT], ld_vgo[LPT];   // ... within a contiguous 64-row tile
 #pragma unroll
   for (int i = 0; i < LPT; ++i) {
     const int r = RPL * (4 * i + wave) + ld_sub;
     ld_row[i] = r;
     ld_koff[i] = (ld_slot ^ (r & (CPR - 1))) << 4;
     ld_voff[i] = (ld_slot ^ ((r & (D == 128 ? 7 : 3)) << 1)) << 4;
+    ld_kgo[i] = r * ROWB + ld_koff[i];
+    ld_vgo[i] = r * ROWB + ld_voff[i];
   }
 
   // First key row of tile t (dense / block lists); kv_len marks "no such block".
@@ -193,7 +200,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
       float* bias = reinterpret_cast<float*>(smem + Cfg::kTotal - Cfg::kBiasBytes) + (t % Cfg::kBiasRing) * 64;
 #pragma unroll
       for (int i = 0; i < LPT; ++i) {
-        dma16(src + (size_t)tok_row[i] * ROWB + (is_v ? ld_voff[i] : ld_koff[i]), slot_base + (4 * i + wave) * 1024);
+        dma16(src, (uint32_t)tok_row[i] * ROWB + (is_v ? ld_voff[i] : ld_koff[i]), slot_base + (4 * i + wave) * 1024);
         if (!is_v && ld_slot == 0) bias[ld_row[i]] = tok_ok[i] ? 0.f : kNegInf;
       }
       if (is_v || !HAS_V) {
@@ -202,11 +209,19 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
       }
     } else {
       const int r0 = tile_row0(t);
+      if (r0 + 64 <= p.kv_len) {
+        // whole tile in range: wave-uniform base, precomputed lane offsets
+        const unsigned char* tb = src + (size_t)r0 * ROWB;
 #pragma unroll
-      for (int i = 0; i < LPT; ++i) {
-        int row = r0 + ld_row[i];
-        row = row > last_row ? last_row : row;
-        dma16(src + (size_t)row * ROWB + (is_v ? ld_voff[i] : ld_koff[i]), slot_base + (4 * i + wave) * 1024);
+        for (int i = 0; i < LPT; ++i) dma16(tb, is_v ? ld_vgo[i] : ld_kgo[i], slot_base + (4 * i + wave) * 1024);
+      } else {
+        // ragged last tile: rows past the end re-read the last row and are masked later
+#pragma unroll
+        for (int i = 0; i < LPT; ++i) {
+          int row = r0 + ld_row[i];
+          row = row > last_row ? last_row : row;
+          dma16(src + (size_t)row * ROWB + (is_v ? ld_voff[i] : ld_koff[i]), slot_base + (4 * i + wave) * 1024);
+        }
       }
     }
   };
@@ -251,7 +266,15 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
 #pragma unroll
   for (int jj = 0; jj < LEAD; ++jj) issue(jj);
 
-  float m_run = kNegInf;   // running raw row max
+  // Softmax state of this lane's query row.  Exponents are taken against a reference
+  // mr_sf (in log2 units, = raw max * sf at the time it was set) that is only moved when
+  // some row of the wave outgrows it by more than kSlack: p = exp2(s*sf - mr_sf) may then
+  // exceed 1 (by at most 2^kSlack), which fp32 sums and bf16 P hold without loss, and the
+  // O / l rescale is skipped on most tiles.  m_true tracks the true raw max for the
+  // statistics outputs.
+  constexpr float kSlack = 8.f;
+  float mr_sf = kNegInf;
+  float m_true = kNegInf;
   float l_run = 0.f;       // running denominator, this lane's keys only
   f32x16 oacc[HAS_V ? NDB : 1];
 #pragma unroll
@@ -261,6 +284,28 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
 
   u32x4 pb[HAS_V ? NKS : 1];
 
+  // Per-lane LDS byte offsets inside a slot; the slot base is added per phase and the
+  // remaining terms are instruction immediates.
+  uint32_t k_lo[NT];       // A operand of QK^T, k-step t, score block 0 (block 1: + 32 rows)
+  {
+    const int krow = ksub * KW + ln;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) k_lo[t] = krow * ROWB + (((2 * t + g) ^ (krow & (CPR - 1))) << 4);
+  }
+  // Transposing V read: in each 16-lane group, lane i addresses 4 dims of key (i>>2);
+  // lane j receives dim j of those 4 keys.  Keys 4g..4g+3 (+8 for the second read) of
+  // each 16-key step, dims 32db + 16*dhalf + 4*(i&3)..+3.
+  uint32_t v_lo[HAS_V ? NDB : 1];
+  if constexpr (HAS_V) {
+    const int i16 = lane & 15;
+    const int dhalf = (lane >> 4) & 1;
+    const int r1 = ksub * KW + 4 * g + (i16 >> 2);
+    const int sw = (r1 & (D == 128 ? 7 : 3)) << 1;
+    const int cb = 2 * dhalf + ((i16 & 3) >> 1);
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) v_lo[db] = r1 * ROWB + (((4 * db + cb) ^ sw) << 4) + ((i16 & 1) << 3);
+  }
+
   for (int it = 0; it < ntiles; ++it) {
     // ================= K phase: S^T = K Q^T, online softmax =================
     const int jk = it * PPT;
@@ -268,19 +313,21 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     __syncthreads();
     issue(jk + LEAD);
     {
-      const unsigned char* kb = smem + (jk % SLOTS) * Cfg::kTileBytes;
+      const uint32_t kb = smem_base + (jk % SLOTS) * Cfg::kTileBytes;
+      u32x4 ka[NMB][NT];
+#pragma unroll
+      for (int mb = 0; mb < NMB; ++mb)
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          ka[mb][t] = *(SPATTN_LDS const u32x4*)(uintptr_t)(kb + k_lo[t] + mb * 32 * ROWB);
+      __builtin_amdgcn_sched_barrier(0);   // all reads in flight before the first multiply
       f32x16 s[NMB];
 #pragma unroll
       for (int mb = 0; mb < NMB; ++mb) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[mb][r] = 0.f;
-        const int krow = ksub * KW + mb * 32 + ln;
-        const unsigned char* krp = kb + krow * ROWB;
 #pragma unroll
-        for (int t = 0; t < NT; ++t) {
-          const u32x4 a = *reinterpret_cast<const u32x4*>(krp + (((2 * t + g) ^ (krow & (CPR - 1))) << 4));
-          s[mb] = mfma32(a, qf[t], s[mb]);
-        }
+        for (int t = 0; t < NT; ++t) s[mb] = mfma32(ka[mb][t], qf[t], s[mb]);
       }
 
       // ---- mask keys that do not exist ----
@@ -317,28 +364,33 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) mloc = fmaxf(mloc, s[mb][r]);
       mloc = fmaxf(mloc, xor32(mloc));
-      const float m_new = fmaxf(m_run, mloc);
-      const float msf = (m_new == kNegInf) ? 0.f : m_new * p.sf;
-      const float alpha = __builtin_amdgcn_exp2f(m_run * p.sf - msf);
-      m_run = m_new;
-      float psum = 0.f;
-#pragma unroll
-      for (int mb = 0; mb < NMB; ++mb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[mb][r], p.sf, -msf));
-          s[mb][r] = e;
-          psum += e;
-        }
-      l_run = l_run * alpha + psum;
-
-      if constexpr (HAS_V) {
-        if (__any(alpha != 1.f)) {
+      m_true = fmaxf(m_true, mloc);
+      const float mloc_sf = mloc * p.sf;
+      if (__any(mloc_sf > mr_sf + kSlack)) {
+        const float new_sf = fmaxf(mr_sf, mloc_sf);
+        const float alpha = (new_sf == kNegInf) ? 1.f : __builtin_amdgcn_exp2f(mr_sf - new_sf);
+        mr_sf = new_sf;
+        l_run *= alpha;
+        if constexpr (HAS_V) {
 #pragma unroll
           for (int db = 0; db < NDB; ++db)
 #pragma unroll
             for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
         }
+      }
+      const float base = (mr_sf == kNegInf) ? 0.f : mr_sf;
+      float psum = 0.f;
+#pragma unroll
+      for (int mb = 0; mb < NMB; ++mb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[mb][r], p.sf, -base));
+          s[mb][r] = e;
+          psum += e;
+        }
+      l_run += psum;
+
+      if constexpr (HAS_V) {
         // P^T operand of k-step ks = 2mb+h: registers 8h..8h+7 of block mb, i.e. keys
         // 32mb + 16h + {4g..4g+3} and 32mb + 16h + 8 + {4g..4g+3}.
 #pragma unroll
@@ -358,33 +410,24 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
       wait_phase(jv);
       __syncthreads();
       issue(jv + LEAD);
-      const unsigned char* vb = smem + (jv % SLOTS) * Cfg::kTileBytes;
-      // Transposing read: in each 16-lane group, lane i addresses 4 dims of key (i>>2);
-      // lane j receives dim j of those 4 keys.
-      const int i16 = lane & 15;
-      const int dhalf = (lane >> 4) & 1;
-      const int rsub = i16 >> 2;                               // key within the group of 4
-      const int cb = 2 * dhalf + ((i16 & 3) >> 1);             // 16-byte chunk within the 32-dim block
-      const int bofs = (i16 & 1) << 3;                         // 8-byte half of the chunk
+      const uint32_t vb = smem_base + (jv % SLOTS) * Cfg::kTileBytes;
+      u32x2 va[NKS][NDB][2];
 #pragma unroll
-      for (int ks = 0; ks < NKS; ++ks) {
-        const int r1 = ksub * KW + 16 * ks + 4 * g + rsub;     // keys of A columns 8g+0..3
-        const int r2 = r1 + 8;                                 // keys of A columns 8g+4..7
-        const int sw1 = (r1 & (D == 128 ? 7 : 3)) << 1;
-        const int sw2 = (r2 & (D == 128 ? 7 : 3)) << 1;
-        const unsigned char* p1 = vb + r1 * ROWB + bofs;
-        const unsigned char* p2 = vb + r2 * ROWB + bofs;
+      for (int ks = 0; ks < NKS; ++ks)
 #pragma unroll
         for (int db = 0; db < NDB; ++db) {
-          const int c = 4 * db + cb;
-          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((SPATTN_LDS s16x4*)(p1 + ((c ^ sw1) << 4)));
-          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((SPATTN_LDS s16x4*)(p2 + ((c ^ sw2) << 4)));
-          const u32x2 lo2 = __builtin_bit_cast(u32x2, lo);
-          const u32x2 hi2 = __builtin_bit_cast(u32x2, hi);
-          const u32x4 a = {lo2[0], lo2[1], hi2[0], hi2[1]};
+          const uint32_t a1 = vb + v_lo[db] + ks * 16 * ROWB;
+          va[ks][db][0] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((SPATTN_LDS s16x4*)(uintptr_t)a1));
+          va[ks][db][1] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((SPATTN_LDS s16x4*)(uintptr_t)(a1 + 8 * ROWB)));
+        }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks)
+#pragma unroll
+        for (int db = 0; db < NDB; ++db) {
+          const u32x4 a = {va[ks][db][0][0], va[ks][db][0][1], va[ks][db][1][0], va[ks][db][1][1]};
           oacc[db] = mfma32(a, pb[ks], oacc[db]);
         }
-      }
     }
   }
   __syncthreads();   // every wave is done with the ring
@@ -392,32 +435,33 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   // ---- combine the two 32-lane halves, then the two key halves -------------------
   float l_tot = l_run + xor32(l_run);
   if constexpr (KSPLIT == 2) {
-    float* mg = reinterpret_cast<float*>(smem) + qsub * ((HAS_V ? D / 2 : 0) + 2) * 64;
+    float* mg = reinterpret_cast<float*>(smem) + qsub * ((HAS_V ? D / 2 : 0) + 3) * 64;
     if (ksub == 1) {
-      mg[lane] = m_run;
+      mg[lane] = mr_sf;
       mg[64 + lane] = l_tot;
+      mg[128 + lane] = m_true;
       if constexpr (HAS_V) {
 #pragma unroll
         for (int db = 0; db < NDB; ++db)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) mg[(2 + db * 16 + r) * 64 + lane] = oacc[db][r];
+          for (int r = 0; r < 16; ++r) mg[(3 + db * 16 + r) * 64 + lane] = oacc[db][r];
       }
     }
     __syncthreads();
     if (ksub == 1) return;
     const float m2 = mg[lane];
     const float l2 = mg[64 + lane];
-    const float m_new = fmaxf(m_run, m2);
-    const float msf = (m_new == kNegInf) ? 0.f : m_new * p.sf;
-    const float a1 = __builtin_amdgcn_exp2f(m_run * p.sf - msf);
-    const float a2 = __builtin_amdgcn_exp2f(m2 * p.sf - msf);
+    m_true = fmaxf(m_true, mg[128 + lane]);
+    const float new_sf = fmaxf(mr_sf, m2);
+    const float a1 = (mr_sf == kNegInf) ? 0.f : __builtin_amdgcn_exp2f(mr_sf - new_sf);
+    const float a2 = (m2 == kNegInf) ? 0.f : __builtin_amdgcn_exp2f(m2 - new_sf);
     l_tot = l_tot * a1 + l2 * a2;
-    m_run = m_new;
+    mr_sf = new_sf;
     if constexpr (HAS_V) {
 #pragma unroll
       for (int db = 0; db < NDB; ++db)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) oacc[db][r] = oacc[db][r] * a1 + mg[(2 + db * 16 + r) * 64 + lane] * a2;
+        for (int r = 0; r < 16; ++r) oacc[db][r] = oacc[db][r] * a1 + mg[(3 + db * 16 + r) * 64 + lane] * a2;
     }
   }
 
@@ -439,15 +483,17 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   }
   if (g == 0) {
     if (p.lse != nullptr && qrow_ok) {
-      p.lse[(size_t)bh * p.S + qrow] = (l_tot > 0.f) ? (m_run * p.scale + __logf(l_tot)) : kNegInf;
+      p.lse[(size_t)bh * p.S + qrow] = (l_tot > 0.f) ? (mr_sf + __log2f(l_tot)) * kLn2 : kNegInf;
     }
     if constexpr (STATS) {
       // Pad rows keep the reference convention max_q = 0, denom = -inf
       // (include/maxq_denom.cuh:202-205).
       if (qrow < p.Sp) {
         const size_t so = (size_t)bh * p.Sp + qrow;
-        p.max_q[so] = (qrow_ok && m_run != kNegInf) ? m_run : 0.f;
-        p.denom[so] = qrow_ok ? l_tot : kNegInf;
+        // the denominator is reported against the true row max
+        const bool any_key = qrow_ok && m_true != kNegInf;
+        p.max_q[so] = any_key ? m_true : 0.f;
+        p.denom[so] = qrow_ok ? (any_key ? l_tot * __builtin_amdgcn_exp2f(mr_sf - m_true * p.sf) : 0.f) : kNegInf;
       }
     }
   }
