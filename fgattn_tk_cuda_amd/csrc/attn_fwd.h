@@ -6,11 +6,10 @@
 //   include/fullattn_wgload_padded.cuh:190-232          (dense attention),
 //   include/maxq_denom_attn.cuh:196-252                 (dense attention + row statistics),
 //   include/maxq_denom.cuh:169-206                      (row statistics only):
-// running raw row max m, p = exp2((s - m) * log2e * scale), fp32 denominator, P rounded
-// to bf16 before PV, O / l at the end.  Keys that do not exist (list position >= n,
-// token id >= kv_len, row >= kv_len) are masked on every tile, a superset of the
-// reference's "NaN row -> -inf on the last tile" (include/asyncloadutils.cuh:124-142,
-// include/pad_utils.cuh:54-75).
+// running row max, p = exp2((s - m) * log2e * scale), fp32 denominator, P rounded to bf16
+// before PV, O / l at the end.  Keys that do not exist (list position >= n, token id >=
+// kv_len, row >= kv_len) are masked on every tile, a superset of the reference's "NaN row
+// -> -inf on the last tile" (include/asyncloadutils.cuh:124-142, include/pad_utils.cuh:54-75).
 //
 // Work split.  A workgroup is 4 waves (256 lanes) and owns one q-block of QBLK rows.
 // Scores are produced transposed, S^T = K Q^T, so that in the 32x32 MFMA accumulator a
@@ -23,42 +22,49 @@
 //
 // Data movement.  K and V tiles (64 rows x D bf16, row-major as in HBM) go HBM -> LDS with
 // global_load_lds_dwordx4: no staging registers, no LDS stores.  Each lane picks which
-// 16-byte chunk of its row it fetches so that the tile lands XOR-swizzled (K: chunk ^
-// row; V: chunk ^ 2*(row&7)).  K is read back as the MFMA A operand with ds_read_b128; the
+// 16-byte chunk of its row it fetches so that the tile lands XOR-swizzled (chunk ^ swz(row),
+// one swizzle for K and V).  K is read back as the MFMA A operand with ds_read_b128; the
 // V^T operand comes from ds_read_b64_tr_b16, which hands lane j of a 16-lane group the
-// j-th 16-bit column of the 4 rows the group addressed.  Tiles live in a ring of kSlots
-// slots consumed in the order K0 V0 K1 V1 ...; every phase is
-//     wait own loads of this phase -> barrier -> issue the load kSlots-1 phases ahead
-//     into the slot the barrier just freed -> multiply,
-// so kSlots-1 tiles are always in flight per workgroup.
+// j-th 16-bit column of the 4 rows the group addressed.
+//
+// Schedule.  Tiles are consumed in "phases" K0 | K1 V0 | K2 V1 | ... : the scores of tile
+// i+1 are multiplied while the softmax of tile i runs on the vector ALU, and the row
+// maxima of tile i+1 are reduced while P_i V_i is multiplied.  Phase j lives in ring slot
+// j & 3; every phase is  wait (own loads of this phase) -> barrier -> issue phase j+3 into
+// the slot the barrier just freed -> multiply.  The steady-state loop is unrolled over two
+// tiles so that every slot is a compile-time constant: LDS addresses are a per-lane base
+// plus an instruction immediate, the wait counts are literals, and the loop carries almost
+// no scalar or address arithmetic - the instruction issue rate, not the matrix pipe, is
+// what bounds this kernel.
 #pragma once
+#include <type_traits>
+
 #include "common.h"
 
 namespace spattn {
 
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 #define SPATTN_LDS __attribute__((address_space(3)))
+typedef SPATTN_LDS const unsigned char* lds_cptr;
 
 template <int D, int MODE, bool HAS_V>
 struct AttnCfg {
   static constexpr int kTileBytes = 64 * D * 2;
-  // D=128: 5 x 16 KB = 80 KB, two workgroups fill the 160 KB of a CU exactly.
-  static constexpr int kSlots = (D == 128) ? (MODE == KV_TOKENS ? 4 : 5) : 8;
-  static constexpr int kLead = kSlots - 1;                 // phases between issue and use
-  static constexpr int kBiasRing = 4;                       // tiles of key-validity bias (token lists)
+  static constexpr int kSlots = 4;
+  static constexpr int kBiasRing = 8;                         // tiles of key-validity bias (token lists)
   static constexpr int kBiasBytes = (MODE == KV_TOKENS) ? kBiasRing * 64 * 4 : 0;
   static constexpr int kRing = kSlots * kTileBytes;
-  static constexpr int kMerge = 2 * (D / 2 + 3) * 64 * 4;   // key-split merge, overlays the ring
+  static constexpr int kMerge = 2 * (D / 2 + 3) * 64 * 4;     // key-split merge, overlays the ring
   static constexpr int kTotal = ((kRing > kMerge) ? kRing : kMerge) + kBiasBytes;
-  static constexpr int kRowsPerLoad = 1024 / (D * 2);       // rows one wave-wide 1 KB load covers
+  static constexpr int kRowsPerLoad = 1024 / (D * 2);         // rows one wave-wide 1 KB load covers
   static constexpr int kLoadsPerTile = kTileBytes / 1024 / 4;   // per wave
 };
 
 // One wave-wide HBM -> LDS copy: lane l's 16 bytes land at lds_base + 16 l.
+// Written as asm on purpose: the compiler does not count this load in its own vmcnt
+// bookkeeping (with the builtin it drains every outstanding load before each LDS read),
+// so the waits are placed by hand.
 __device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_base) {
-  // Written as asm on purpose: the compiler does not count this load in its own vmcnt
-  // bookkeeping (with the builtin it drains every outstanding load before each LDS read),
-  // so the waits below are placed by hand.
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(gptr) : "memory");
 }
 // Same with a wave-uniform base pointer and a 32-bit per-lane byte offset.
@@ -81,18 +87,16 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   constexpr int NMB = KW / 32;       // 32-key score blocks per wave
   constexpr int NT = D / 16;         // k-steps of the QK^T product
   constexpr int NDB = D / 32;        // 32-wide blocks of the head dim
-  constexpr int NKS = KW / 16;       // k-steps of the PV product
   constexpr int CPR = D / 8;         // 16-byte chunks per row
   constexpr int ROWB = D * 2;        // bytes per row
-  constexpr int SLOTS = Cfg::kSlots;
-  constexpr int LEAD = Cfg::kLead;
+  constexpr int TILE = Cfg::kTileBytes;
   constexpr int LPT = Cfg::kLoadsPerTile;
   constexpr int RPL = Cfg::kRowsPerLoad;
-  constexpr int PPT = HAS_V ? 2 : 1;   // phases per tile
   constexpr float kNegInf = -__builtin_huge_valf();
 
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-  const uint32_t smem_base = (uint32_t)(uintptr_t)(SPATTN_LDS unsigned char*)smem;
+  const lds_cptr smem_l = (lds_cptr)smem;
+  const uint32_t smem_base = (uint32_t)(uintptr_t)smem_l;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -128,24 +132,24 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     n = n < 0 ? 0 : (n > p.idx_stride ? p.idx_stride : n);
     ntiles = (MODE == KV_TOKENS) ? ((n + 63) >> 6) : n;
   }
-  const int nphase = ntiles * PPT;
   const int last_row = p.kv_len - 1;
+  // Phase numbers: with V, 0 = K0, 2i+1 = K(i+1), 2i+2 = V(i); phase 2*ntiles-1 would be a
+  // K tile past the end and is never issued.  Without V, phase j = K(j).
+  const int last_phase = HAS_V ? 2 * ntiles : ntiles - 1;
 
   // ---- loader role: load i of a tile covers rows RPL*(4i + wave) .. +RPL-1 ----------
   const int ld_sub = lane / CPR;       // row within the load
   const int ld_slot = lane % CPR;      // 16-byte position within the row in LDS
-  int ld_row[LPT];
-  int ld_koff[LPT], ld_voff[LPT];      // byte offset of this lane's chunk within its row
-  uint32_t ld_kgo[LPT], ld_vgo[LPT];   // ... within a contiguous 64-row tile
+  // Row r of a tile stores its 16-byte chunk c at position c ^ swz(r).  Eight consecutive
+  // rows put one chunk into eight different 16-byte bank groups (the K reads), four
+  // consecutive rows put one 32-byte window into four different windows (the transposing
+  // V reads), and rows r and r+8 share a swizzle.
+  auto swz = [](int r) -> int { return D == 128 ? ((r & 7) << 1) : (((r & 3) << 1) | ((r >> 2) & 1)); };
+  auto ld_row = [&](int i) -> int { return RPL * (4 * i + wave) + ld_sub; };
+  auto ld_off = [&](int i) -> int { return (ld_slot ^ swz(ld_row(i))) << 4; };   // chunk offset within the row
+  uint32_t ld_go[LPT];                 // lane offset within a contiguous 64-row tile
 #pragma unroll
-  for (int i = 0; i < LPT; ++i) {
-    const int r = RPL * (4 * i + wave) + ld_sub;
-    ld_row[i] = r;
-    ld_koff[i] = (ld_slot ^ (r & (CPR - 1))) << 4;
-    ld_voff[i] = (ld_slot ^ ((r & (D == 128 ? 7 : 3)) << 1)) << 4;
-    ld_kgo[i] = r * ROWB + ld_koff[i];
-    ld_vgo[i] = r * ROWB + ld_voff[i];
-  }
+  for (int i = 0; i < LPT; ++i) ld_go[i] = ld_row(i) * ROWB + ld_off(i);
 
   // First key row of tile t (dense / block lists); kv_len marks "no such block".
   auto tile_row0 = [&](int t) -> int {
@@ -159,9 +163,12 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
 
   // Token lists: the RPL token ids behind one load are wave-uniform, so they are fetched
   // as scalars (tok_raw) one tile ahead and turned into this lane's row (tok_row) just
-  // before the K and V loads of that tile are issued.
+  // before the K load of that tile is issued; V tiles are issued one tile later and take
+  // their rows from a two-deep queue.
   int tok_raw[MODE == KV_TOKENS ? LPT : 1][MODE == KV_TOKENS ? RPL : 1];
-  int tok_row[MODE == KV_TOKENS ? LPT : 1];
+  int tok_row[MODE == KV_TOKENS ? LPT : 1];      // rows of the next K tile to issue
+  int tok_row_v0[MODE == KV_TOKENS ? LPT : 1];   // rows of the next V tile to issue
+  int tok_row_v1[MODE == KV_TOKENS ? LPT : 1];   // rows of the V tile after that
   bool tok_ok[MODE == KV_TOKENS ? LPT : 1];
   auto tok_fetch = [&](int t) {
     if constexpr (MODE == KV_TOKENS) {
@@ -179,31 +186,37 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
 #pragma unroll
         for (int s = 0; s < RPL; ++s) {
           int v = tok_raw[i][s];
-          asm volatile("" : "+s"(v));   // keep it a scalar: no per-lane reload of the list
+          v = __builtin_amdgcn_readfirstlane(v);   // keeps the list a scalar load (no per-lane reload)
           tok = (ld_sub == s) ? v : tok;
         }
-        tok_ok[i] = (t * 64 + ld_row[i]) < n && (unsigned)tok <= (unsigned)last_row;
+        tok_ok[i] = (t * 64 + ld_row(i)) < n && (unsigned)tok <= (unsigned)last_row;
         tok_row[i] = tok_ok[i] ? tok : 0;
       }
     }
   };
 
-  // Issue the loads of phase jj (tile jj / PPT; K if even or no V, else V).  Phases are
-  // issued strictly in order, which the token-id prefetch relies on.
-  auto issue = [&](int jj) {
-    if (jj >= nphase) return;
-    const int t = HAS_V ? (jj >> 1) : jj;
-    const bool is_v = HAS_V && (jj & 1);
-    const uint32_t slot_base = smem_base + (uint32_t)(jj % SLOTS) * Cfg::kTileBytes;
+  // Loads of one K or V tile into ring slot `slot`.  Issue order is K0 K1 V0 K2 V1 ...,
+  // which the token-row queue relies on.
+  auto issue_tile = [&](int t, int slot, bool is_v) {
+    const uint32_t slot_base = smem_base + (uint32_t)slot * TILE;
     const unsigned char* src = is_v ? vh : kh;
     if constexpr (MODE == KV_TOKENS) {
       float* bias = reinterpret_cast<float*>(smem + Cfg::kTotal - Cfg::kBiasBytes) + (t % Cfg::kBiasRing) * 64;
 #pragma unroll
       for (int i = 0; i < LPT; ++i) {
-        dma16(src, (uint32_t)tok_row[i] * ROWB + (is_v ? ld_voff[i] : ld_koff[i]), slot_base + (4 * i + wave) * 1024);
-        if (!is_v && ld_slot == 0) bias[ld_row[i]] = tok_ok[i] ? 0.f : kNegInf;
+        const int row = is_v ? tok_row_v0[i] : tok_row[i];
+        dma16(src, (uint32_t)row * ROWB + ld_off(i), slot_base + (4 * i + wave) * 1024);
+        if (!is_v && ld_slot == 0) bias[ld_row(i)] = tok_ok[i] ? 0.f : kNegInf;
       }
-      if (is_v || !HAS_V) {
+      if (is_v) {
+#pragma unroll
+        for (int i = 0; i < LPT; ++i) tok_row_v0[i] = tok_row_v1[i];
+      } else {
+#pragma unroll
+        for (int i = 0; i < LPT; ++i) {
+          if (t == 0) tok_row_v0[i] = tok_row[i];
+          tok_row_v1[i] = tok_row[i];
+        }
         tok_resolve(t + 1);
         tok_fetch(t + 2);
       }
@@ -213,35 +226,40 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
         // whole tile in range: wave-uniform base, precomputed lane offsets
         const unsigned char* tb = src + (size_t)r0 * ROWB;
 #pragma unroll
-        for (int i = 0; i < LPT; ++i) dma16(tb, is_v ? ld_vgo[i] : ld_kgo[i], slot_base + (4 * i + wave) * 1024);
+        for (int i = 0; i < LPT; ++i) dma16(tb, ld_go[i], slot_base + (4 * i + wave) * 1024);
       } else {
         // ragged last tile: rows past the end re-read the last row and are masked later
 #pragma unroll
         for (int i = 0; i < LPT; ++i) {
-          int row = r0 + ld_row[i];
+          int row = r0 + ld_row(i);
           row = row > last_row ? last_row : row;
-          dma16(src + (size_t)row * ROWB + (is_v ? ld_voff[i] : ld_koff[i]), slot_base + (4 * i + wave) * 1024);
+          dma16(src + (size_t)row * ROWB + ld_off(i), slot_base + (4 * i + wave) * 1024);
         }
       }
     }
   };
-
-  // Wait until this wave's loads of phase j have landed: everything issued after them
-  // (up to LEAD-1 phases) may stay in flight.
-  auto wait_phase = [&](int j) {
-    const int later = nphase - 1 - j;   // phases issued after j
-    if (later >= LEAD - 1) {
-      wait_vmcnt<(LEAD - 1) * LPT>();
+  auto phase_exists = [&](int j) -> bool {
+    if (j > last_phase) return false;
+    if constexpr (HAS_V) return j != 2 * ntiles - 1;
+    return true;
+  };
+  // Generic form: issue phase j if it exists.
+  auto issue_phase = [&](int j) {
+    if (!phase_exists(j)) return;
+    if constexpr (HAS_V) {
+      if (j == 0) issue_tile(0, 0, false);
+      else if (j & 1) issue_tile((j + 1) / 2, j & 3, false);
+      else issue_tile(j / 2 - 1, j & 3, true);
     } else {
-      // tail: fewer loads behind this one
-      if constexpr (LEAD - 1 > 6) if (later == 6) { wait_vmcnt<6 * LPT>(); return; }
-      if constexpr (LEAD - 1 > 5) if (later == 5) { wait_vmcnt<5 * LPT>(); return; }
-      if constexpr (LEAD - 1 > 4) if (later == 4) { wait_vmcnt<4 * LPT>(); return; }
-      if constexpr (LEAD - 1 > 3) if (later == 3) { wait_vmcnt<3 * LPT>(); return; }
-      if constexpr (LEAD - 1 > 2) if (later == 2) { wait_vmcnt<2 * LPT>(); return; }
-      if constexpr (LEAD - 1 > 1) if (later == 1) { wait_vmcnt<1 * LPT>(); return; }
-      wait_vmcnt<0>();
+      issue_tile(j, j & 3, false);
     }
+  };
+  // Generic wait for phase j: phases j+1 and j+2, if they exist, may stay in flight.
+  auto wait_generic = [&](int j) {
+    const int later = (phase_exists(j + 1) ? 1 : 0) + (phase_exists(j + 2) ? 1 : 0);
+    if (later == 2) wait_vmcnt<2 * LPT>();
+    else if (later == 1) wait_vmcnt<LPT>();
+    else wait_vmcnt<0>();
   };
 
   // ---- prologue ------------------------------------------------------------------
@@ -263,8 +281,9 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   tok_fetch(0);
   tok_resolve(0);
   tok_fetch(1);
-#pragma unroll
-  for (int jj = 0; jj < LEAD; ++jj) issue(jj);
+  issue_phase(0);
+  issue_phase(1);
+  issue_phase(2);
 
   // Softmax state of this lane's query row.  Exponents are taken against a reference
   // mr_sf (in log2 units, = raw max * sf at the time it was set) that is only moved when
@@ -282,152 +301,244 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
 
-  u32x4 pb[HAS_V ? NKS : 1];
+  u32x4 pb[HAS_V ? 2 * NMB : 1];   // P^T operands, k-step 2mb + h
 
-  // Per-lane LDS byte offsets inside a slot; the slot base is added per phase and the
-  // remaining terms are instruction immediates.
-  uint32_t k_lo[NT];       // A operand of QK^T, k-step t, score block 0 (block 1: + 32 rows)
+  // Per-lane LDS addresses inside slot 0; slot, score block and k-step offsets are added
+  // as constants (instruction immediates in the unrolled loop).
+  lds_cptr k_lo[NT];       // A operand of QK^T, k-step t, score block 0
   {
     const int krow = ksub * KW + ln;
 #pragma unroll
-    for (int t = 0; t < NT; ++t) k_lo[t] = krow * ROWB + (((2 * t + g) ^ (krow & (CPR - 1))) << 4);
+    for (int t = 0; t < NT; ++t) k_lo[t] = smem_l + krow * ROWB + (((2 * t + g) ^ swz(krow)) << 4);
   }
   // Transposing V read: in each 16-lane group, lane i addresses 4 dims of key (i>>2);
   // lane j receives dim j of those 4 keys.  Keys 4g..4g+3 (+8 for the second read) of
   // each 16-key step, dims 32db + 16*dhalf + 4*(i&3)..+3.
-  uint32_t v_lo[HAS_V ? NDB : 1];
+  lds_cptr v_lo[HAS_V ? NDB : 1];
   if constexpr (HAS_V) {
     const int i16 = lane & 15;
     const int dhalf = (lane >> 4) & 1;
     const int r1 = ksub * KW + 4 * g + (i16 >> 2);
-    const int sw = (r1 & (D == 128 ? 7 : 3)) << 1;
+    const int sw = swz(r1);   // also the swizzle of row r1 + 8, the second read
     const int cb = 2 * dhalf + ((i16 & 3) >> 1);
 #pragma unroll
-    for (int db = 0; db < NDB; ++db) v_lo[db] = r1 * ROWB + (((4 * db + cb) ^ sw) << 4) + ((i16 & 1) << 3);
+    for (int db = 0; db < NDB; ++db) v_lo[db] = smem_l + r1 * ROWB + (((4 * db + cb) ^ sw) << 4) + ((i16 & 1) << 3);
   }
 
-  for (int it = 0; it < ntiles; ++it) {
-    // ================= K phase: S^T = K Q^T, online softmax =================
-    const int jk = it * PPT;
-    wait_phase(jk);
-    __syncthreads();
-    issue(jk + LEAD);
-    {
-      const uint32_t kb = smem_base + (jk % SLOTS) * Cfg::kTileBytes;
-      u32x4 ka[NMB][NT];
+  // ---- building blocks --------------------------------------------------------------
+  // Keys of tile `it` that do not exist get -inf.  Accumulator register 4j+i of block mb
+  // is key ksub*KW + 32mb + 8j + 4g + i of the tile.
+  auto mask_tile = [&](int it, f32x16 (&s)[NMB]) {
+    if constexpr (MODE == KV_TOKENS) {
+      const float* bias = reinterpret_cast<const float*>(smem + Cfg::kTotal - Cfg::kBiasBytes) + (it % Cfg::kBiasRing) * 64;
 #pragma unroll
       for (int mb = 0; mb < NMB; ++mb)
 #pragma unroll
-        for (int t = 0; t < NT; ++t)
-          ka[mb][t] = *(SPATTN_LDS const u32x4*)(uintptr_t)(kb + k_lo[t] + mb * 32 * ROWB);
-      __builtin_amdgcn_sched_barrier(0);   // all reads in flight before the first multiply
-      f32x16 s[NMB];
-#pragma unroll
-      for (int mb = 0; mb < NMB; ++mb) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) s[mb][r] = 0.f;
-#pragma unroll
-        for (int t = 0; t < NT; ++t) s[mb] = mfma32(ka[mb][t], qf[t], s[mb]);
-      }
-
-      // ---- mask keys that do not exist ----
-      // Accumulator register 4j+i of block mb is key ksub*KW + 32mb + 8j + 4g + i of the tile.
-      if constexpr (MODE == KV_TOKENS) {
-        const float* bias = reinterpret_cast<const float*>(smem + Cfg::kTotal - Cfg::kBiasBytes) + (it % Cfg::kBiasRing) * 64;
+        for (int j = 0; j < 4; ++j) {
+          const float4 bv = *reinterpret_cast<const float4*>(bias + ksub * KW + 32 * mb + 8 * j + 4 * g);
+          s[mb][4 * j + 0] += bv.x;
+          s[mb][4 * j + 1] += bv.y;
+          s[mb][4 * j + 2] += bv.z;
+          s[mb][4 * j + 3] += bv.w;
+        }
+    } else {
+      const int r0 = tile_row0(it);
+      if (r0 + 64 > p.kv_len) {
 #pragma unroll
         for (int mb = 0; mb < NMB; ++mb)
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const float4 bv = *reinterpret_cast<const float4*>(bias + ksub * KW + 32 * mb + 8 * j + 4 * g);
-            s[mb][4 * j + 0] += bv.x;
-            s[mb][4 * j + 1] += bv.y;
-            s[mb][4 * j + 2] += bv.z;
-            s[mb][4 * j + 3] += bv.w;
+          for (int r = 0; r < 16; ++r) {
+            const int key = r0 + ksub * KW + 32 * mb + 8 * (r >> 2) + 4 * g + (r & 3);
+            if (key >= p.kv_len) s[mb][r] = kNegInf;
           }
-      } else {
-        const int r0 = tile_row0(it);
-        if (r0 + 64 > p.kv_len) {
-#pragma unroll
-          for (int mb = 0; mb < NMB; ++mb)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const int key = r0 + ksub * KW + 32 * mb + 8 * (r >> 2) + 4 * g + (r & 3);
-              if (key >= p.kv_len) s[mb][r] = kNegInf;
-            }
-        }
-      }
-
-      // ---- online softmax; one query row per lane ----
-      float mloc = s[0][0];
-#pragma unroll
-      for (int mb = 0; mb < NMB; ++mb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) mloc = fmaxf(mloc, s[mb][r]);
-      mloc = fmaxf(mloc, xor32(mloc));
-      m_true = fmaxf(m_true, mloc);
-      const float mloc_sf = mloc * p.sf;
-      if (__any(mloc_sf > mr_sf + kSlack)) {
-        const float new_sf = fmaxf(mr_sf, mloc_sf);
-        const float alpha = (new_sf == kNegInf) ? 1.f : __builtin_amdgcn_exp2f(mr_sf - new_sf);
-        mr_sf = new_sf;
-        l_run *= alpha;
-        if constexpr (HAS_V) {
-#pragma unroll
-          for (int db = 0; db < NDB; ++db)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
-        }
-      }
-      const float base = (mr_sf == kNegInf) ? 0.f : mr_sf;
-      float psum = 0.f;
-#pragma unroll
-      for (int mb = 0; mb < NMB; ++mb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[mb][r], p.sf, -base));
-          s[mb][r] = e;
-          psum += e;
-        }
-      l_run += psum;
-
-      if constexpr (HAS_V) {
-        // P^T operand of k-step ks = 2mb+h: registers 8h..8h+7 of block mb, i.e. keys
-        // 32mb + 16h + {4g..4g+3} and 32mb + 16h + 8 + {4g..4g+3}.
-#pragma unroll
-        for (int ks = 0; ks < NKS; ++ks) {
-          const int mb = ks >> 1, h8 = (ks & 1) * 8;
-          pb[ks][0] = pack_bf16(s[mb][h8 + 0], s[mb][h8 + 1]);
-          pb[ks][1] = pack_bf16(s[mb][h8 + 2], s[mb][h8 + 3]);
-          pb[ks][2] = pack_bf16(s[mb][h8 + 4], s[mb][h8 + 5]);
-          pb[ks][3] = pack_bf16(s[mb][h8 + 6], s[mb][h8 + 7]);
-        }
       }
     }
-
-    // ================= V phase: O^T += V^T P^T =================
+  };
+  // Row max of a score tile (both 32-lane halves); returns max * sf.
+  auto row_stats = [&](const f32x16 (&s)[NMB]) -> float {
+    float mloc = s[0][0];
+#pragma unroll
+    for (int mb = 0; mb < NMB; ++mb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mloc = fmaxf(mloc, s[mb][r]);
+    mloc = fmaxf(mloc, xor32(mloc));
+    m_true = fmaxf(m_true, mloc);
+    return mloc * p.sf;
+  };
+  // Move the exponent reference if some row of the wave outgrew it; rescales O and l.
+  auto maybe_rescale = [&](float mloc_sf) {
+    if (__any(mloc_sf > mr_sf + kSlack)) {
+      const float new_sf = fmaxf(mr_sf, mloc_sf);
+      const float alpha = (new_sf == kNegInf) ? 1.f : __builtin_amdgcn_exp2f(mr_sf - new_sf);
+      mr_sf = new_sf;
+      l_run *= alpha;
+      if constexpr (HAS_V) {
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+      }
+    }
+  };
+  // p = exp2(s*sf - reference) for registers r0..r0+cnt-1 of block mb; adds to the row sum
+  // and leaves P^T as bf16 MFMA operands (k-step 2mb+h takes registers 8h..8h+7 of block
+  // mb, i.e. keys 32mb + 16h + {4g..4g+3} and 32mb + 16h + 8 + {4g..4g+3}).
+  auto softmax_chunk = [&](f32x16 (&s)[NMB], float base, int mb, int r0, int cnt) {
+#pragma unroll
+    for (int r = r0; r < r0 + cnt; r += 2) {
+      const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[mb][r], p.sf, -base));
+      const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[mb][r + 1], p.sf, -base));
+      l_run += e0;
+      l_run += e1;
+      if constexpr (HAS_V) pb[2 * mb + (r >> 3)][(r & 7) >> 1] = pack_bf16(e0, e1);
+    }
+  };
+  // Pin the softmax results where they are produced; otherwise the compiler sinks the
+  // whole softmax to the first use of P, behind the next barrier, and nothing overlaps
+  // the MFMAs.
+  auto pin_softmax = [&]() {
+    asm volatile("" : "+v"(l_run));
     if constexpr (HAS_V) {
-      const int jv = jk + 1;
-      wait_phase(jv);
-      __syncthreads();
-      issue(jv + LEAD);
-      const uint32_t vb = smem_base + (jv % SLOTS) * Cfg::kTileBytes;
-      u32x2 va[NKS][NDB][2];
 #pragma unroll
-      for (int ks = 0; ks < NKS; ++ks)
+      for (int ks = 0; ks < 2 * NMB; ++ks)
 #pragma unroll
-        for (int db = 0; db < NDB; ++db) {
-          const uint32_t a1 = vb + v_lo[db] + ks * 16 * ROWB;
-          va[ks][db][0] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((SPATTN_LDS s16x4*)(uintptr_t)a1));
-          va[ks][db][1] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((SPATTN_LDS s16x4*)(uintptr_t)(a1 + 8 * ROWB)));
+        for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(pb[ks][i]));
+    }
+  };
+  auto softmax_only = [&](f32x16 (&s)[NMB]) {
+    const float base = (mr_sf == kNegInf) ? 0.f : mr_sf;
+#pragma unroll
+    for (int mb = 0; mb < NMB; ++mb) softmax_chunk(s, base, mb, 0, 16);
+  };
+  // s_out^T = K Q^T from the K tile at ring offset kofs (bytes), one 32-key block at a
+  // time; if WITH_SM, the softmax of s_in is interleaved: one MFMA, then the vector-ALU
+  // work of 16/NT score registers.
+  auto qk_tile = [&](auto with_sm, uint32_t kofs, f32x16 (&s_out)[NMB], f32x16 (&s_in)[NMB]) {
+    constexpr bool WITH_SM = decltype(with_sm)::value;
+    constexpr int EPM = 16 / NT;
+    const float base = (mr_sf == kNegInf) ? 0.f : mr_sf;
+#pragma unroll
+    for (int mb = 0; mb < NMB; ++mb) {
+      u32x4 ka[NT];
+#pragma unroll
+      for (int t = 0; t < NT; ++t) ka[t] = *(SPATTN_LDS const u32x4*)(k_lo[t] + kofs + mb * 32 * ROWB);
+      __builtin_amdgcn_sched_barrier(0);   // all reads in flight before the first multiply
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s_out[mb][r] = 0.f;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        s_out[mb] = mfma32(ka[t], qf[t], s_out[mb]);
+        if constexpr (WITH_SM) softmax_chunk(s_in, base, mb, t * EPM, EPM);
+      }
+      if constexpr (WITH_SM) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);            // one MFMA
+          __builtin_amdgcn_sched_group_barrier(0x002, EPM * 7 / 2, 0);  // its share of the softmax
         }
+      }
       __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (WITH_SM) pin_softmax();
+  };
+  // O^T += V^T P^T from the V tile at ring offset vofs, two 16-key steps at a time.
+  auto pv_tile = [&](uint32_t vofs) {
+    if constexpr (HAS_V) {
 #pragma unroll
-      for (int ks = 0; ks < NKS; ++ks)
+      for (int mb = 0; mb < NMB; ++mb) {
+        u32x2 va[2][NDB][2];
 #pragma unroll
-        for (int db = 0; db < NDB; ++db) {
-          const u32x4 a = {va[ks][db][0][0], va[ks][db][0][1], va[ks][db][1][0], va[ks][db][1][1]};
-          oacc[db] = mfma32(a, pb[ks], oacc[db]);
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int db = 0; db < NDB; ++db) {
+            const lds_cptr a1 = v_lo[db] + vofs + (2 * mb + h) * 16 * ROWB;
+            va[h][db][0] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((SPATTN_LDS s16x4*)a1));
+            va[h][db][1] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((SPATTN_LDS s16x4*)(a1 + 8 * ROWB)));
+          }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int db = 0; db < NDB; ++db) {
+            const u32x4 a = {va[h][db][0][0], va[h][db][0][1], va[h][db][1][0], va[h][db][1][1]};
+            oacc[db] = mfma32(a, pb[2 * mb + h], oacc[db]);
+          }
+      }
+    }
+  };
+
+  // One tile of the pipeline: K phase of tile it+1 (ring slot KS) with the softmax of tile
+  // it (scores in s_a), then V phase of tile it (ring slot VS) with the row maxima of tile
+  // it+1 (scores in s_b).  In the steady state every later phase exists, so waits and
+  // issues are unconditional.
+  auto tile_body = [&](auto ks_c, auto vs_c, auto steady_c, int it, f32x16 (&s_a)[NMB], f32x16 (&s_b)[NMB]) {
+    constexpr int KS = decltype(ks_c)::value;
+    constexpr int VS = decltype(vs_c)::value;
+    constexpr bool STEADY = decltype(steady_c)::value;
+    {
+      const int j = HAS_V ? 2 * it + 1 : it + 1;
+      if constexpr (STEADY) wait_vmcnt<2 * LPT>(); else wait_generic(j);
+      __syncthreads();
+      if constexpr (HAS_V) {
+        if (STEADY || it + 1 < ntiles) issue_tile(it + 1, (VS + 2) & 3, true);     // phase j+3 = V(it+1)
+      } else {
+        if (STEADY || it + 4 < ntiles) issue_tile(it + 4, (KS + 3) & 3, false);    // phase j+3 = K(it+4)
+      }
+      qk_tile(std::true_type{}, KS * TILE, s_b, s_a);
+      mask_tile(it + 1, s_b);
+    }
+    if constexpr (HAS_V) {
+      const int j = 2 * it + 2;
+      if constexpr (STEADY) wait_vmcnt<2 * LPT>(); else wait_generic(j);
+      __syncthreads();
+      if (STEADY || it + 3 < ntiles) issue_tile(it + 3, KS, false);                // phase j+3 = K(it+3)
+      pv_tile(VS * TILE);
+    }
+    maybe_rescale(row_stats(s_b));
+  };
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  using I2 = std::integral_constant<int, 2>;
+  using I3 = std::integral_constant<int, 3>;
+
+  if (ntiles > 0) {
+    f32x16 s_e[NMB], s_o[NMB];   // scores of even / odd tiles
+    // phase 0: scores of tile 0
+    wait_generic(0);
+    __syncthreads();
+    issue_phase(3);
+    qk_tile(std::false_type{}, 0, s_e, s_e);
+    mask_tile(0, s_e);
+    maybe_rescale(row_stats(s_e));
+
+    int it = 0;
+    if constexpr (HAS_V) {
+      // tile `it` has its next K tile in slot (2it+1)&3 and its V tile in slot (2it+2)&3
+      for (; it + 4 < ntiles; it += 2) {
+        tile_body(I1{}, I2{}, std::true_type{}, it, s_e, s_o);
+        tile_body(I3{}, I0{}, std::true_type{}, it + 1, s_o, s_e);
+      }
+      for (; it + 1 < ntiles; ++it) {
+        if (it & 1) tile_body(I3{}, I0{}, std::false_type{}, it, s_o, s_e);
+        else tile_body(I1{}, I2{}, std::false_type{}, it, s_e, s_o);
+      }
+      if (it & 1) softmax_only(s_o); else softmax_only(s_e);
+      wait_vmcnt<0>();
+      __syncthreads();
+      pv_tile((uint32_t)((2 * ntiles) & 3) * TILE);
+    } else {
+      // tile it+1 sits in K slot (it+1)&3
+      for (; it + 1 < ntiles; ++it) {
+        switch ((it + 1) & 3) {
+          case 0: tile_body(I0{}, I0{}, std::false_type{}, it, s_e, s_o); break;
+          case 1: tile_body(I1{}, I0{}, std::false_type{}, it, s_e, s_o); break;
+          case 2: tile_body(I2{}, I0{}, std::false_type{}, it, s_e, s_o); break;
+          default: tile_body(I3{}, I0{}, std::false_type{}, it, s_e, s_o); break;
         }
+#pragma unroll
+        for (int mb = 0; mb < NMB; ++mb) s_e[mb] = s_o[mb];
+      }
+      softmax_only(s_e);
     }
   }
   __syncthreads();   // every wave is done with the ring
