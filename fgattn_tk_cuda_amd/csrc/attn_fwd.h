@@ -195,17 +195,25 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     }
   };
 
-  // Loads of one K or V tile into ring slot `slot`.  Issue order is K0 K1 V0 K2 V1 ...,
-  // which the token-row queue relies on.
-  auto issue_tile = [&](int t, int slot, bool is_v) {
-    const uint32_t slot_base = smem_base + (uint32_t)slot * TILE;
+  // Loads of one K or V tile into ring slot `slot`: prepare() resolves the wave-uniform
+  // base and this lane's byte offsets, load(i) issues the i-th of the LPT wave-wide copies.
+  // Issue order of the tiles is K0 K1 V0 K2 V1 ..., which the token-row queue relies on.
+  struct TileLoad {
+    const unsigned char* base;
+    uint32_t lds;
+    uint32_t go[LPT];
+  };
+  auto prepare_tile = [&](int t, int slot, bool is_v) -> TileLoad {
+    TileLoad tl;
+    tl.lds = smem_base + (uint32_t)slot * TILE + wave * 1024;
     const unsigned char* src = is_v ? vh : kh;
     if constexpr (MODE == KV_TOKENS) {
+      tl.base = src;
       float* bias = reinterpret_cast<float*>(smem + Cfg::kTotal - Cfg::kBiasBytes) + (t % Cfg::kBiasRing) * 64;
 #pragma unroll
       for (int i = 0; i < LPT; ++i) {
         const int row = is_v ? tok_row_v0[i] : tok_row[i];
-        dma16(src, (uint32_t)row * ROWB + ld_off(i), slot_base + (4 * i + wave) * 1024);
+        tl.go[i] = (uint32_t)row * ROWB + ld_off(i);
         if (!is_v && ld_slot == 0) bias[ld_row(i)] = tok_ok[i] ? 0.f : kNegInf;
       }
       if (is_v) {
@@ -223,20 +231,27 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     } else {
       const int r0 = tile_row0(t);
       if (r0 + 64 <= p.kv_len) {
-        // whole tile in range: wave-uniform base, precomputed lane offsets
-        const unsigned char* tb = src + (size_t)r0 * ROWB;
+        tl.base = src + (size_t)r0 * ROWB;   // whole tile in range
 #pragma unroll
-        for (int i = 0; i < LPT; ++i) dma16(tb, ld_go[i], slot_base + (4 * i + wave) * 1024);
+        for (int i = 0; i < LPT; ++i) tl.go[i] = ld_go[i];
       } else {
         // ragged last tile: rows past the end re-read the last row and are masked later
+        tl.base = src;
 #pragma unroll
         for (int i = 0; i < LPT; ++i) {
           int row = r0 + ld_row(i);
           row = row > last_row ? last_row : row;
-          dma16(src + (size_t)row * ROWB + ld_off(i), slot_base + (4 * i + wave) * 1024);
+          tl.go[i] = (uint32_t)row * ROWB + ld_off(i);
         }
       }
     }
+    return tl;
+  };
+  auto load_part = [&](const TileLoad& tl, int i) { dma16(tl.base, tl.go[i], tl.lds + i * 4096); };
+  auto issue_tile = [&](int t, int slot, bool is_v) {
+    const TileLoad tl = prepare_tile(t, slot, is_v);
+#pragma unroll
+    for (int i = 0; i < LPT; ++i) load_part(tl, i);
   };
   auto phase_exists = [&](int j) -> bool {
     if (j > last_phase) return false;
@@ -361,7 +376,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     for (int mb = 0; mb < NMB; ++mb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) mloc = fmaxf(mloc, s[mb][r]);
-    mloc = fmaxf(mloc, xor32(mloc));
+    mloc = pair_max(mloc);
     m_true = fmaxf(m_true, mloc);
     return mloc * p.sf;
   };
@@ -413,7 +428,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   // s_out^T = K Q^T from the K tile at ring offset kofs (bytes), one 32-key block at a
   // time; if WITH_SM, the softmax of s_in is interleaved: one MFMA, then the vector-ALU
   // work of 16/NT score registers.
-  auto qk_tile = [&](auto with_sm, uint32_t kofs, f32x16 (&s_out)[NMB], f32x16 (&s_in)[NMB]) {
+  auto qk_tile = [&](auto with_sm, uint32_t kofs, f32x16 (&s_out)[NMB], f32x16 (&s_in)[NMB], const TileLoad* tl) {
     constexpr bool WITH_SM = decltype(with_sm)::value;
     constexpr int EPM = 16 / NT;
     const float base = (mr_sf == kNegInf) ? 0.f : mr_sf;
@@ -429,6 +444,13 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
       for (int t = 0; t < NT; ++t) {
         s_out[mb] = mfma32(ka[t], qf[t], s_out[mb]);
         if constexpr (WITH_SM) softmax_chunk(s_in, base, mb, t * EPM, EPM);
+        // the next tile's copies are spread over the multiplies: issued in one burst they
+        // queue behind the other waves' copies and stall this wave
+        if (tl != nullptr) {
+          constexpr int STEP = (NMB * NT) / LPT;
+          const int m = mb * NT + t;
+          if (m % STEP == STEP - 1) load_part(*tl, m / STEP);
+        }
       }
       if constexpr (WITH_SM) {
 #pragma unroll
@@ -442,7 +464,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     if constexpr (WITH_SM) pin_softmax();
   };
   // O^T += V^T P^T from the V tile at ring offset vofs, two 16-key steps at a time.
-  auto pv_tile = [&](uint32_t vofs) {
+  auto pv_tile = [&](uint32_t vofs, const TileLoad* tl) {
     if constexpr (HAS_V) {
 #pragma unroll
       for (int mb = 0; mb < NMB; ++mb) {
@@ -462,6 +484,11 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
           for (int db = 0; db < NDB; ++db) {
             const u32x4 a = {va[h][db][0][0], va[h][db][0][1], va[h][db][1][0], va[h][db][1][1]};
             oacc[db] = mfma32(a, pb[2 * mb + h], oacc[db]);
+            if (tl != nullptr) {   // the next tile's copies, spread over the multiplies
+              constexpr int STEP = (NMB * 2 * NDB) / LPT;
+              const int m = (mb * 2 + h) * NDB + db;
+              if (m % STEP == STEP - 1) load_part(*tl, m / STEP);
+            }
           }
       }
     }
@@ -479,20 +506,32 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
       const int j = HAS_V ? 2 * it + 1 : it + 1;
       if constexpr (STEADY) wait_vmcnt<2 * LPT>(); else wait_generic(j);
       __syncthreads();
-      if constexpr (HAS_V) {
-        if (STEADY || it + 1 < ntiles) issue_tile(it + 1, (VS + 2) & 3, true);     // phase j+3 = V(it+1)
+      // phase j+3 is V(it+1) (with V) or K(it+4)
+      if constexpr (STEADY) {
+        const TileLoad tl = HAS_V ? prepare_tile(it + 1, (VS + 2) & 3, true) : prepare_tile(it + 4, (KS + 3) & 3, false);
+        qk_tile(std::true_type{}, KS * TILE, s_b, s_a, &tl);
       } else {
-        if (STEADY || it + 4 < ntiles) issue_tile(it + 4, (KS + 3) & 3, false);    // phase j+3 = K(it+4)
+        if constexpr (HAS_V) {
+          if (it + 1 < ntiles) issue_tile(it + 1, (VS + 2) & 3, true);
+        } else {
+          if (it + 4 < ntiles) issue_tile(it + 4, (KS + 3) & 3, false);
+        }
+        qk_tile(std::true_type{}, KS * TILE, s_b, s_a, nullptr);
       }
-      qk_tile(std::true_type{}, KS * TILE, s_b, s_a);
       mask_tile(it + 1, s_b);
     }
     if constexpr (HAS_V) {
       const int j = 2 * it + 2;
       if constexpr (STEADY) wait_vmcnt<2 * LPT>(); else wait_generic(j);
       __syncthreads();
-      if (STEADY || it + 3 < ntiles) issue_tile(it + 3, KS, false);                // phase j+3 = K(it+3)
-      pv_tile(VS * TILE);
+      // phase j+3 is K(it+3)
+      if constexpr (STEADY) {
+        const TileLoad tl = prepare_tile(it + 3, KS, false);
+        pv_tile(VS * TILE, &tl);
+      } else {
+        if (it + 3 < ntiles) issue_tile(it + 3, KS, false);
+        pv_tile(VS * TILE, nullptr);
+      }
     }
     maybe_rescale(row_stats(s_b));
   };
@@ -507,7 +546,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     wait_generic(0);
     __syncthreads();
     issue_phase(3);
-    qk_tile(std::false_type{}, 0, s_e, s_e);
+    qk_tile(std::false_type{}, 0, s_e, s_e, nullptr);
     mask_tile(0, s_e);
     maybe_rescale(row_stats(s_e));
 
@@ -525,7 +564,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
       if (it & 1) softmax_only(s_o); else softmax_only(s_e);
       wait_vmcnt<0>();
       __syncthreads();
-      pv_tile((uint32_t)((2 * ntiles) & 3) * TILE);
+      pv_tile((uint32_t)((2 * ntiles) & 3) * TILE, nullptr);
     } else {
       // tile it+1 sits in K slot (it+1)&3
       for (; it + 1 < ntiles; ++it) {
@@ -544,7 +583,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   __syncthreads();   // every wave is done with the ring
 
   // ---- combine the two 32-lane halves, then the two key halves -------------------
-  float l_tot = l_run + xor32(l_run);
+  float l_tot = pair_sum(l_run);
   if constexpr (KSPLIT == 2) {
     float* mg = reinterpret_cast<float*>(smem) + qsub * ((HAS_V ? D / 2 : 0) + 3) * 64;
     if (ksub == 1) {

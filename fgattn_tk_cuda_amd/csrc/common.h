@@ -53,8 +53,26 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, b);
 }
 
-// Value held by lane ^ 32.
-__device__ __forceinline__ float xor32(float x) { return __shfl_xor(x, 32, 64); }
+// Max / sum of the values held by lanes l and l ^ 32, in both lanes.  v_permlane32_swap
+// exchanges the upper half of its first operand with the lower half of its second: with
+// the same value in both, each lane ends up holding its own and its partner's value.
+// Written as asm: both operands are read and written, and the wait states cover a
+// preceding vector-ALU write of either operand.
+__device__ __forceinline__ void pair_values(float x, float& lo, float& hi) {
+  lo = x;
+  hi = x;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(lo), "+v"(hi));
+}
+__device__ __forceinline__ float pair_max(float x) {
+  float a, b;
+  pair_values(x, a, b);
+  return fmaxf(a, b);
+}
+__device__ __forceinline__ float pair_sum(float x) {
+  float a, b;
+  pair_values(x, a, b);
+  return a + b;
+}
 
 // WGs are dealt to the 8 XCDs round-robin by launch order; give each XCD one
 // contiguous range of logical work ids so that neighbouring q-blocks of a head
