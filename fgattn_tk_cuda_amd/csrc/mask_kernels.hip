@@ -144,55 +144,84 @@ hipError_t run_booleanmask(int* mask, float thresh, int mask_stride, const float
 // booleanmask_to_indexmask.  Reference: include/mask_utils.cuh:273-302 - for each
 // (b,h,q-block) row: count = #{c < kv_len : mask[c] > 0}, list = those c, entries past the
 // count keep the caller's fill.  The reference appends through one global atomic per key
-// (order undefined); here one wave owns one row, reads it as 16-byte vectors, ranks every
-// kept key with wave ballots and writes the list in ascending order - no atomics, no LDS,
-// no barrier, and the result is deterministic.  The kernel is a pure HBM stream:
-// 4 bytes read per mask entry, 4 bytes written per kept key.
+// (order undefined); here one wave owns one row and streams it as 16-byte vectors with the
+// next 8 KB already in flight.  Every kept key is ranked with wave ballots and appended to
+// a per-wave LDS ring, which is written out in ascending order 1 KB at a time - no
+// atomics, no barrier, full-line stores, and the result is deterministic.  The kernel is
+// a pure HBM stream: 4 bytes read per mask entry, 4 bytes written per kept key.
 // ------------------------------------------------------------------------------------
-constexpr int kCompactUnroll = 8;   // 16-byte loads in flight per lane
+constexpr int kCompactUnroll = 8;      // 16-byte loads per lane per step (8 KB per wave)
+constexpr int kCompactRing = 1024;     // ints in the per-wave output ring (>= 256 pending + 256*... see flush)
 
 __global__ __launch_bounds__(256) void compact_kernel(int* __restrict__ kv_indices, int* __restrict__ kv_num,
                                                       const int* __restrict__ mask, int rows, int mask_stride,
                                                       int kv_len) {
+  constexpr int U = kCompactUnroll;
+  constexpr int SPAN = 256 * U;        // ints per wave step
+  constexpr int QN = kCompactRing;
+  __shared__ __attribute__((aligned(16))) int ring[4][QN];
   const int lane = threadIdx.x & 63;
-  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int wave = threadIdx.x >> 6;
+  const int row = blockIdx.x * 4 + wave;
   if (row >= rows) return;
   const int* __restrict__ src = mask + (size_t)row * mask_stride;
   int* __restrict__ dst = kv_indices + (size_t)row * mask_stride;
+  int* q = ring[wave];
   const int lim = kv_len < mask_stride ? kv_len : mask_stride;
-  int base = 0;
-  constexpr int kSpan = 64 * 4 * kCompactUnroll;   // ints per wave iteration
-  for (int c0 = 0; c0 < lim; c0 += kSpan) {
-    i32x4 val[kCompactUnroll];
+  const int nstep = (lim + SPAN - 1) / SPAN;
+  int tail = 0;   // keys appended to the ring so far
+  int head = 0;   // keys written out so far
+
+  i32x4 cur[U], nxt[U];
+  // mask_stride is a multiple of 4, so a vector that starts below lim stays inside the row
+  auto load = [&](int c, i32x4 (&v)[U]) {
 #pragma unroll
-    for (int u = 0; u < kCompactUnroll; ++u) {
-      const int e0 = c0 + u * 256 + 4 * lane;
+    for (int u = 0; u < U; ++u) {
+      const int e0 = c * SPAN + u * 256 + 4 * lane;
       const i32x4 z = {0, 0, 0, 0};
-      val[u] = (e0 < lim) ? __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(src + e0)) : z;
+      v[u] = (e0 < lim) ? __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(src + e0)) : z;
     }
+  };
+  auto process = [&](int c, const i32x4 (&v)[U]) {
+    const bool full = (c + 1) * SPAN <= lim;   // no entry of this step reaches lim
 #pragma unroll
-    for (int u = 0; u < kCompactUnroll; ++u) {
-      const int e0 = c0 + u * 256 + 4 * lane;
+    for (int u = 0; u < U; ++u) {
+      const int e0 = c * SPAN + u * 256 + 4 * lane;
       bool f[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) f[i] = (e0 + i < lim) && (val[u][i] > 0);
+      for (int i = 0; i < 4; ++i) f[i] = v[u][i] > 0 && (full || e0 + i < lim);
       const unsigned long long b0 = __ballot(f[0]), b1 = __ballot(f[1]), b2 = __ballot(f[2]), b3 = __ballot(f[3]);
-      if ((b0 | b1 | b2 | b3) == 0ull) continue;
       // keys of lower lanes come first, then this lane's own lower keys
-      int pos = base;
+      int pos = tail;
       pos = __builtin_amdgcn_mbcnt_hi((unsigned)(b0 >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)b0, pos));
       pos = __builtin_amdgcn_mbcnt_hi((unsigned)(b1 >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)b1, pos));
       pos = __builtin_amdgcn_mbcnt_hi((unsigned)(b2 >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)b2, pos));
       pos = __builtin_amdgcn_mbcnt_hi((unsigned)(b3 >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)b3, pos));
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        if (f[i]) dst[pos] = e0 + i;
+        if (f[i]) q[pos & (QN - 1)] = e0 + i;
         pos += f[i] ? 1 : 0;
       }
-      base += __popcll(b0) + __popcll(b1) + __popcll(b2) + __popcll(b3);
+      tail += __popcll(b0) + __popcll(b1) + __popcll(b2) + __popcll(b3);
+      // at most 255 keys were pending and at most 256 were added: the ring never wraps
+      // onto unwritten keys; head stays a multiple of 256, so the stores are whole lines
+      while (tail - head >= 256) {
+        *reinterpret_cast<i32x4*>(dst + head + 4 * lane) = *reinterpret_cast<const i32x4*>(q + ((head + 4 * lane) & (QN - 1)));
+        head += 256;
+      }
     }
+  };
+
+  if (nstep > 0) load(0, cur);
+  for (int c = 0; c < nstep; ++c) {
+    if (c + 1 < nstep) load(c + 1, nxt);
+    process(c, cur);
+#pragma unroll
+    for (int u = 0; u < U; ++u) cur[u] = nxt[u];
   }
-  if (lane == 0) kv_num[row] = base;
+  for (; head < tail; head += 64)
+    if (head + lane < tail) dst[head + lane] = q[(head + lane) & (QN - 1)];
+  if (lane == 0) kv_num[row] = tail;
 }
 
 hipError_t run_compact(int* kv_indices, int* kv_num, const int* mask, int rows, int mask_stride, int kv_len,
