@@ -1,0 +1,260 @@
+"""Mask helpers of the reference's ``spattn/mask_utils.py`` over the gfx950 operators.
+
+Same names, argument meaning and tensor conventions as the reference
+(python/spattn/mask_utils.py); the pure-torch functions are the semantic definition of
+the masks, the ``*_cuda`` functions run the device operators.  Differences kept on
+purpose: tensors are created on the device of their inputs instead of a hard-coded
+'cuda', and ``seq`` of ``bitmask_to_indexmask_cuda`` defaults to the mask width instead
+of a stale constant.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import cuda_attn  # noqa: F401  (loading it registers torch.ops.cuda_attn)
+
+spattn_interface = torch.ops.cuda_attn
+
+BLOCKSZ = 128   # q-block of the threshold pre-pass (python/spattn/mask_utils.py:249,312)
+
+
+def _padded(seq: int, blk: int = BLOCKSZ) -> int:
+    return blk * ((seq + blk - 1) // blk)
+
+
+# ----------------------------------------------------------------------------------
+# mask caches (python/spattn/mask_utils.py:17-98)
+# ----------------------------------------------------------------------------------
+class NaiveMaskCache:
+    """Index lists per layer, recomputed on the diffusion steps in ``compute_cache_at``."""
+
+    def __init__(self, compute_cache_at):
+        self.cache = {}
+        self.compute_cache_at = compute_cache_at
+
+    def run_fullattn(self, ditrun):
+        return ditrun in self.compute_cache_at
+
+    def get_mask_from_cache(self, layer):
+        return self.cache[layer]
+
+    def update_cache(self, layer, kv_indices, kv_num_indices):
+        self.cache[layer] = (kv_indices, kv_num_indices)
+
+
+class OffloadMaskCache(NaiveMaskCache):
+    """Keeps the index lists in host memory between uses."""
+
+    def get_mask_from_cache(self, layer, ditrun=0):
+        kv_indices, kv_num_indices = self.cache[layer]
+        return kv_indices.to(kv_num_indices.device), kv_num_indices
+
+    def update_cache(self, layer, kv_indices, kv_num_indices):
+        self.cache[layer] = (kv_indices.cpu(), kv_num_indices)
+
+
+class BitMaskCache:
+    """Stores the vote mask and re-expands it to index lists on every use."""
+
+    def __init__(self, compute_cache_at):
+        self.cache = {}
+        self.compute_cache_at = compute_cache_at
+
+    def run_fullattn(self, ditrun):
+        return ditrun in self.compute_cache_at
+
+    def get_mask_from_cache(self, layer):
+        mask, seq_len = self.cache[layer]
+        return bitmask_to_indexmask_cuda(mask, seq_len)
+
+    def update_cache(self, layer, bytemask, seq_len):
+        self.cache[layer] = (bytemask, seq_len)
+
+
+class CompressedBitMaskCache(BitMaskCache):
+    """Stores the mask bit-packed (8 keys per byte, least significant bit first)."""
+
+    def get_mask_from_cache(self, layer):
+        packed, seq_len = self.cache[layer]
+        return bitmask_to_indexmask_cuda(unpack(packed).to(torch.int32), seq_len)
+
+    def update_cache(self, layer, bitmask, seq_len):
+        self.cache[layer] = (pack(bitmask > 0), seq_len)
+
+
+# ----------------------------------------------------------------------------------
+# 2-D attention-map helpers (python/spattn/mask_utils.py:107-167)
+# ----------------------------------------------------------------------------------
+def _pool_rows(attnmap, block, reduce):
+    rows, cols = attnmap.shape
+    pad = (-rows) % block
+    if pad:
+        # a ragged last block is reduced over the rows it has: pad with copies of the last row
+        attnmap = torch.cat([attnmap, attnmap[-1:].expand(pad, cols)], dim=0)
+    return reduce(attnmap.view(-1, block, cols), 1)
+
+
+def attnmapand(attnmap, BLOCK_SZ=128):
+    """min over each block of BLOCK_SZ rows (python/spattn/mask_utils.py:107-123)."""
+    return _pool_rows(attnmap, BLOCK_SZ, lambda t, d: t.min(dim=d).values)
+
+
+def attnmapor(attnmap, BLOCK_SZ=128):
+    """max over each block of BLOCK_SZ rows (python/spattn/mask_utils.py:126-142)."""
+    return _pool_rows(attnmap, BLOCK_SZ, lambda t, d: t.max(dim=d).values)
+
+
+def attnmapbroadcast(attnmapand_, BLOCK_SZ=128):
+    """Repeat every row BLOCK_SZ times (python/spattn/mask_utils.py:145-149)."""
+    return attnmapand_.repeat_interleave(BLOCK_SZ, dim=0)
+
+
+def boolean_to_index_mask_2d(boolean_mask):
+    """Rows of a boolean [R,N] mask -> ascending column lists padded with N, and counts
+    (python/spattn/mask_utils.py:152-167)."""
+    rows, n = boolean_mask.shape
+    keep = boolean_mask != 0
+    # a stable sort moves the kept columns to the front in ascending order
+    order = torch.sort((~keep).to(torch.uint8), dim=1, stable=True).indices
+    counts = keep.sum(dim=1)
+    col = torch.arange(n, device=boolean_mask.device).expand(rows, n)
+    index_mask = torch.where(col < counts[:, None], order, torch.full_like(order, n))
+    return index_mask.to(torch.int32), counts.to(torch.int32)
+
+
+# ----------------------------------------------------------------------------------
+# index lists (python/spattn/mask_utils.py:175-203)
+# ----------------------------------------------------------------------------------
+def allindex_mask(B, H, max_stride, S, BLOCKSZ, device="cuda"):
+    nb = (S + BLOCKSZ - 1) // BLOCKSZ
+    kv_indices = torch.arange(max_stride, device=device, dtype=torch.int32).expand(B, H, nb, max_stride).contiguous()
+    return kv_indices, torch.full((B, H, nb), S, device=device, dtype=torch.int32)
+
+
+def halfindex_mask(B, H, S, BLOCKSZ, device="cuda"):
+    nb = (S + BLOCKSZ - 1) // BLOCKSZ
+    kv_indices = (2 * torch.arange(S // 2, device=device, dtype=torch.int32)).expand(B, H, nb, S // 2).contiguous()
+    return kv_indices, torch.full((B, H, nb), S // 2, device=device, dtype=torch.int32)
+
+
+def allindex_randompermutation_mask(B, H, max_stride, S, BLOCKSZ, device="cuda"):
+    nb = (S + BLOCKSZ - 1) // BLOCKSZ
+    row = torch.full((max_stride,), max_stride, device=device, dtype=torch.int32)
+    row[:S] = torch.randperm(S, device=device).to(torch.int32)
+    return row.expand(B, H, nb, max_stride).contiguous(), torch.full((B, H, nb), S, device=device, dtype=torch.int32)
+
+
+# ----------------------------------------------------------------------------------
+# pure-torch definition of the threshold mask (python/spattn/mask_utils.py:206-245)
+# ----------------------------------------------------------------------------------
+def qk_bitmask(q, k, thresh=0.001, blocksz=128):
+    """mask[b,h,I,c] = any row r of q-block I has softmax(q k^T / sqrt(D))[r,c] > thresh."""
+    B, H, S, D = q.shape
+    out = []
+    for b in range(B):
+        per_head = []
+        for h in range(H):
+            p = torch.softmax((q[b, h] @ k[b, h].T) * (D ** -0.5), dim=-1)
+            per_head.append(attnmapor(p > thresh, blocksz))
+        out.append(torch.stack(per_head))
+    return torch.stack(out)
+
+
+def bitmask_to_indexmask(booleanmask):
+    B, H, SB, MS = booleanmask.shape
+    idx, cnt = boolean_to_index_mask_2d(booleanmask.reshape(B * H * SB, MS))
+    return idx.view(B, H, SB, MS), cnt.view(B, H, SB)
+
+
+def qk_indexmask(q, k, thresh=0.001, blocksz=128):
+    return bitmask_to_indexmask(qk_bitmask(q, k, thresh, blocksz))
+
+
+# ----------------------------------------------------------------------------------
+# device path (python/spattn/mask_utils.py:248-382)
+# ----------------------------------------------------------------------------------
+def _stats_buffers(q):
+    B, H, S, _ = q.shape
+    sp = _padded(S)
+    max_q = torch.empty((B, H, 1, sp), dtype=torch.float32, device=q.device)
+    denom = torch.empty((B, H, 1, sp), dtype=torch.float32, device=q.device)
+    return max_q, denom
+
+
+def qk_bitmask_from_maxq_denom_cuda(max_q, denom, q, k, thresh, blocksz=128):
+    """Vote mask int32 [B,H,ceil(S/128),Sp] from row statistics (python/spattn/mask_utils.py:337-355)."""
+    assert blocksz == BLOCKSZ
+    B, H, S, _ = q.shape
+    booleanmask = torch.zeros((B, H, (S + blocksz - 1) // blocksz, max_q.shape[3]), dtype=torch.int32, device=q.device)
+    spattn_interface.booleanmask_128(booleanmask, max_q.contiguous(), denom.contiguous(), q.contiguous(), k.contiguous(), thresh)
+    return booleanmask
+
+
+def qk_bitmask_cuda(q, k, thresh, blocksz=128):
+    """Boolean mask via maxq_denom + booleanmask_128 (python/spattn/mask_utils.py:248-269)."""
+    assert blocksz == BLOCKSZ
+    max_q, denom = _stats_buffers(q)
+    spattn_interface.maxq_denom(max_q, denom, q.contiguous(), k.contiguous())
+    return qk_bitmask_from_maxq_denom_cuda(max_q, denom, q, k, thresh, blocksz) > 0
+
+
+def bitmask_to_indexmask_cuda(booleanmask, seq=None):
+    """Index lists (ascending, padded with mask_stride) and counts from a vote mask
+    (python/spattn/mask_utils.py:293-303); ``seq`` is the kv length."""
+    B, H, SB, MS = booleanmask.shape
+    if seq is None:
+        seq = MS
+    kv_indices = torch.full((B, H, SB, MS), MS, dtype=torch.int32, device=booleanmask.device)
+    num_kv_indices = torch.zeros((B, H, SB), dtype=torch.int32, device=booleanmask.device)
+    spattn_interface.booleanmask_to_indexmask(kv_indices, num_kv_indices, booleanmask.to(torch.int32).contiguous(), seq)
+    return kv_indices, num_kv_indices
+
+
+def qk_indexmask_from_maxq_denom_cuda(max_q, denom, q, k, thresh, blocksz=128):
+    """python/spattn/mask_utils.py:358-382."""
+    booleanmask = qk_bitmask_from_maxq_denom_cuda(max_q, denom, q, k, thresh, blocksz)
+    return bitmask_to_indexmask_cuda(booleanmask, q.shape[2])
+
+
+def qk_indexmask_cuda(q, k, thresh, blocksz=128):
+    """Statistics -> vote mask -> index lists (python/spattn/mask_utils.py:306-334)."""
+    assert blocksz == BLOCKSZ
+    max_q, denom = _stats_buffers(q)
+    spattn_interface.maxq_denom(max_q, denom, q.contiguous(), k.contiguous())
+    return qk_indexmask_from_maxq_denom_cuda(max_q, denom, q, k, thresh, blocksz)
+
+
+def qk_lshmask_indices(query, key, thresh, blocksz=128):
+    raise NotImplementedError   # as in the reference (python/spattn/mask_utils.py:385-386)
+
+
+def qk_topkmask_indices(q, k, select_k, blocksz=128):
+    """Top-k keys per q-block by (block-mean query) . key (python/spattn/mask_utils.py:389-417)."""
+    B, H, S, D = q.shape
+    nb = (S + blocksz - 1) // blocksz
+    pad = nb * blocksz - S
+    qf = q.float()
+    if pad:
+        qf = torch.cat([qf, torch.zeros((B, H, pad, D), device=q.device)], dim=2)
+    rows = torch.full((nb,), float(blocksz), device=q.device)
+    rows[-1] = blocksz - pad
+    qmean = qf.view(B, H, nb, blocksz, D).sum(dim=3) / rows[None, None, :, None]
+    score = torch.einsum("bhmd,bhnd->bhmn", qmean * (D ** -0.5), k.float())
+    kv_indices = torch.topk(score, select_k, dim=-1, sorted=True).indices.to(torch.int32)
+    return kv_indices, torch.full((B, H, nb), select_k, device=q.device, dtype=torch.int32)
+
+
+# ----------------------------------------------------------------------------------
+# bit packing (python/spattn/mask_utils.py:421-439)
+# ----------------------------------------------------------------------------------
+def pack(bool_tensor):
+    """8 booleans -> one uint8, least significant bit first; the last dim must be a multiple of 8."""
+    w = torch.tensor([1, 2, 4, 8, 16, 32, 64, 128], dtype=torch.uint8, device=bool_tensor.device)
+    grouped = bool_tensor.reshape(*bool_tensor.shape[:-1], bool_tensor.shape[-1] // 8, 8).to(torch.uint8)
+    return (grouped * w).sum(dim=-1).to(torch.uint8)
+
+
+def unpack(packed_tensor):
+    w = torch.tensor([1, 2, 4, 8, 16, 32, 64, 128], dtype=torch.uint8, device=packed_tensor.device)
+    bits = (packed_tensor.unsqueeze(-1) & w) != 0
+    return bits.reshape(*packed_tensor.shape[:-1], packed_tensor.shape[-1] * 8)

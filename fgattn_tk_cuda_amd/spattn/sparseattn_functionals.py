@@ -1,0 +1,125 @@
+"""Model-facing attention functions of the reference's ``spattn/sparseattn_functionals.py``.
+
+Each takes ``(query, key, value, current_layer, ditrun, **kwargs)`` with bf16 tensors
+[B,H,S,D] and returns the bf16 output, like the reference
+(python/spattn/sparseattn_functionals.py:10-154).  Outputs are allocated on the device
+of ``query``.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import mask_utils
+from . import cuda_attn  # noqa: F401
+
+spattn_interface = torch.ops.cuda_attn
+
+
+def _out_like(query):
+    return torch.empty(query.shape, device=query.device, dtype=torch.bfloat16)
+
+
+def _c(*tensors):
+    return tuple(t.contiguous() for t in tensors)
+
+
+def baseline_attn(query, key, value, current_layer=None, ditrun=None, *args, **kwargs):
+    """Dense attention (python/spattn/sparseattn_functionals.py:10-15)."""
+    out = _out_like(query)
+    spattn_interface.full_attn(out, *_c(query, key, value))
+    return out
+
+
+def _dense_with_stats(query, key, value):
+    out = _out_like(query)
+    max_q, denom = mask_utils._stats_buffers(query)
+    spattn_interface.fullattn_maxq_denom(out, max_q, denom, *_c(query, key, value))
+    return out, max_q, denom
+
+
+def baseline_attn_maxq_denom(query, key, value, current_layer=None, ditrun=None, *args, **kwargs):
+    """Dense attention through the fused statistics kernel (:18-26)."""
+    return _dense_with_stats(query, key, value)[0]
+
+
+def _sparse(query, key, value, kv_indices, kv_num_indices):
+    out = _out_like(query)
+    spattn_interface.sp_attn(out, *_c(query, key, value, kv_indices, kv_num_indices))
+    return out
+
+
+def attn_computed_with_sparse_mask_python(query, key, value, current_layer=None, ditrun=None, *args, **kwargs):
+    """Index lists from the pure-torch mask definition, then sparse attention (:29-36)."""
+    kv_indices, kv_num_indices = mask_utils.qk_indexmask(query, key, kwargs["thresh"], blocksz=kwargs["blocksz"])
+    return _sparse(query, key, value, kv_indices, kv_num_indices)
+
+
+def attn_topkmask_cuda(query, key, value, current_layer=None, ditrun=None, *args, **kwargs):
+    """Top-k key lists per q-block, then sparse attention (:39-48).  The sparse operator
+    needs lists padded to a multiple of 128 keys."""
+    select_k = kwargs.get("select_k") or query.shape[2]
+    kv_indices, kv_num_indices = mask_utils.qk_topkmask_indices(query, key, select_k, blocksz=kwargs["blocksz"])
+    stride = mask_utils._padded(select_k)
+    if stride != select_k:
+        pad = torch.full((*kv_indices.shape[:3], stride - select_k), stride, dtype=torch.int32, device=query.device)
+        kv_indices = torch.cat([kv_indices, pad], dim=-1)
+    return _sparse(query, key, value, kv_indices, kv_num_indices)
+
+
+def attn_computed_with_sparse_mask_cuda(query, key, value, *args, **kwargs):
+    """Threshold pre-pass on the device, then sparse attention (:62-70)."""
+    kv_indices, kv_num_indices = mask_utils.qk_indexmask_cuda(query, key, kwargs["thresh"], blocksz=kwargs["blocksz"])
+    return _sparse(query, key, value, kv_indices, kv_num_indices)
+
+
+def compute_cache_and_attn_cuda(query, key, value, *args, **kwargs):
+    """Dense attention plus the index lists for later steps (:75-85)."""
+    out, max_q, denom = _dense_with_stats(query, key, value)
+    kv_indices, kv_num_indices = mask_utils.qk_indexmask_from_maxq_denom_cuda(
+        max_q, denom, query, key, kwargs["thresh"], blocksz=kwargs["blocksz"])
+    return out, kv_indices, kv_num_indices
+
+
+def sparse_attn_from_cache_cuda(query, key, value, *args, **kwargs):
+    """Sparse attention from cached lists (:88-93)."""
+    kv_indices, kv_num_indices = kwargs["mask_cache"].get_mask_from_cache(kwargs.get("current_layer"))
+    return _sparse(query, key, value, kv_indices, kv_num_indices)
+
+
+def cached_attn_cuda(query, key, value, current_layer, ditrun, *args, **kwargs):
+    """On the steps that refresh the cache: dense attention with statistics, then the mask
+    pre-pass; on every other step: sparse attention from the cached lists (:95-114)."""
+    mask_cache = kwargs["mask_cache"]
+    if mask_cache.run_fullattn(ditrun):
+        out, max_q, denom = _dense_with_stats(query, key, value)
+        kv_indices, kv_num_indices = mask_utils.qk_indexmask_from_maxq_denom_cuda(
+            max_q, denom, query, key, kwargs["thresh"], blocksz=kwargs["blocksz"])
+        mask_cache.update_cache(current_layer, kv_indices, kv_num_indices)
+        return out
+    kv_indices, kv_num_indices = mask_cache.get_mask_from_cache(current_layer)
+    return _sparse(query, key, value, kv_indices, kv_num_indices)
+
+
+def bitmaskcached_attn_cuda(query, key, value, current_layer, ditrun, *args, **kwargs):
+    """Like cached_attn_cuda with the vote mask (not the lists) kept in the cache (:117-134)."""
+    mask_cache = kwargs["mask_cache"]
+    if mask_cache.run_fullattn(ditrun):
+        out, max_q, denom = _dense_with_stats(query, key, value)
+        bitmask = mask_utils.qk_bitmask_from_maxq_denom_cuda(max_q, denom, query, key, kwargs["thresh"], blocksz=kwargs["blocksz"])
+        mask_cache.update_cache(current_layer, bitmask, query.shape[2])
+        return out
+    kv_indices, kv_num_indices = mask_cache.get_mask_from_cache(current_layer)
+    return _sparse(query, key, value, kv_indices, kv_num_indices)
+
+
+def attn_2xmask_cuda(query, key, value, current_layer=None, ditrun=None, *args, **kwargs):
+    """Every second key (:137-154)."""
+    B, H, S, _ = query.shape
+    blocksz = kwargs["blocksz"]
+    nb = (S + blocksz - 1) // blocksz
+    stride = mask_utils._padded(S)
+    row = torch.full((stride,), stride, dtype=torch.int32, device=query.device)
+    row[: S // 2] = 2 * torch.arange(S // 2, dtype=torch.int32, device=query.device)
+    kv_indices = row.expand(B, H, nb, stride).contiguous()
+    kv_num_indices = torch.full((B, H, nb), S // 2, dtype=torch.int32, device=query.device)
+    return _sparse(query, key, value, kv_indices, kv_num_indices)

@@ -1,0 +1,153 @@
+"""GPU: the benchmark configurations at (or near) full size, checked through properties
+that do not need a full-size oracle run: sampled q-blocks against the oracle, agreement of
+the two entry points, bitwise repeatability, and the pre-pass round trip."""
+import numpy as np
+import pytest
+import torch
+
+from fgattn_tk_cuda_amd import capi, workloads as wl
+from oracle import spattn_oracle as orc
+from helpers import assert_close_o, assert_close_stat, f32, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def _oracle_block_rows(q, k, v, bi, bc, b, h, i, qblk, S):
+    """Oracle O and lse for q-block i of head (b,h) from its block list (the oracle's own
+    softmax on the gathered keys; avoids a full-size oracle call)."""
+    D = q.shape[-1]
+    blocks = bi[b, h, i, : int(bc[b, h, i])].numpy().astype(np.int64)
+    lst = (blocks[:, None] * 64 + np.arange(64)[None]).reshape(-1)
+    lst = lst[lst < S]
+    r = slice(i * qblk, min(S, (i + 1) * qblk))
+    scale = 1.0 / np.sqrt(D)
+    s = f32(q[b, h, r]) @ f32(k[b, h])[lst].T
+    p, den, m = orc._softmax_rows(s, scale, True)
+    return (p @ f32(v[b, h])[lst]) / den[:, None], m * np.float32(scale) + np.log(den)
+
+
+def test_cfg3_headline_shape(dev):
+    """B=2 H=32 N=16384 d=128, 26 of 256 blocks per 64-row q-block."""
+    print("case cfg3 full size", flush=True)
+    c = wl.CONFIGS["cfg3_sparse_16k"]
+    B, H, S, D, qblk = c["B"], c["H"], c["S"], c["D"], c["qblk"]
+    q, k, v = wl.randn_qkv(B, H, S, D, seed=0)
+    bi, bc = wl.uniform_block_lists(B, H, S, qblk, 64, 26, seed=1)
+    qd, kd, vd, bid, bcd = to_dev(dev, q, k, v, bi, bc)
+    o = torch.full_like(qd, float("nan"))
+    lse = torch.full((B, H, S), float("nan"), device=dev)
+    capi.sp_attn_blocks(o, qd, kd, vd, bid, bcd, lse=lse, qblk=qblk)
+    torch.cuda.synchronize()
+    assert torch.isfinite(o.float()).all() and torch.isfinite(lse).all()
+    rng = np.random.default_rng(2)
+    for _ in range(12):
+        b, h, i = int(rng.integers(B)), int(rng.integers(H)), int(rng.integers(S // qblk))
+        wo, wlse = _oracle_block_rows(q, k, v, bi, bc, b, h, i, qblk, S)
+        r = slice(i * qblk, (i + 1) * qblk)
+        assert_close_o(f32(o[b, h, r]), wo, "cfg3 q-block (%d,%d,%d)" % (b, h, i))
+        assert_close_stat(f32(lse[b, h, r]), wlse, "cfg3 lse")
+    # bitwise repeatable: no atomics anywhere in the kernel
+    o2 = torch.empty_like(o)
+    capi.sp_attn_blocks(o2, qd, kd, vd, bid, bcd, qblk=qblk)
+    assert torch.equal(o.view(torch.int16), o2.view(torch.int16))
+    # the token-list operator on the same lists (one head, to bound the index tensor)
+    tok, num = wl.blocks_to_tokens(bi[:1, :1], bc[:1, :1], S)
+    o3 = torch.empty_like(qd[:1, :1])
+    capi.sp_attn(o3, qd[:1, :1].contiguous(), kd[:1, :1].contiguous(), vd[:1, :1].contiguous(), tok.to(dev), num.to(dev), qblk=qblk)
+    assert_close_o(f32(o3), f32(o[:1, :1]), "token path vs block path")
+
+
+def test_cfg2_dense_shape(dev):
+    print("case cfg2 full size", flush=True)
+    c = wl.CONFIGS["cfg2_dense"]
+    B, H, S, D = c["B"], c["H"], c["S"], c["D"]
+    q, k, v = to_dev(dev, *wl.randn_qkv(B, H, S, D, seed=3))
+    o = torch.empty_like(q)
+    capi.full_attn(o, q, k, v)
+    want = torch.nn.functional.scaled_dot_product_attention(q[:, :4].float(), k[:, :4].float(), v[:, :4].float())
+    assert_close_o(f32(o[:, :4]), f32(want), "cfg2 vs SDPA")
+    want = torch.nn.functional.scaled_dot_product_attention(q[:, 12:].float(), k[:, 12:].float(), v[:, 12:].float())
+    assert_close_o(f32(o[:, 12:]), f32(want), "cfg2 vs SDPA (last heads)")
+
+
+def test_cfg5_zipf_lists(dev):
+    """Skewed per-row counts, q-block 128, kv-block 64 (two heads of the 64K configuration's shape, N=16384)."""
+    print("case cfg5 zipf", flush=True)
+    B, H, S, D, qblk = 1, 2, 16384, 128, 128
+    q, k, v = wl.randn_qkv(B, H, S, D, seed=4)
+    counts = wl.zipf_counts(B, H, S // qblk, s=1.2, lo=1, hi=256, seed=5)
+    bi, bc = wl.ragged_block_lists(B, H, S, qblk, 64, counts, seed=6)
+    qd, kd, vd, bid, bcd = to_dev(dev, q, k, v, bi, bc)
+    o = torch.full_like(qd, float("nan"))
+    lse = torch.full((B, H, S), float("nan"), device=dev)
+    capi.sp_attn_blocks(o, qd, kd, vd, bid, bcd, lse=lse, qblk=qblk)
+    assert torch.isfinite(o.float()).all()
+    order = np.argsort(counts.reshape(-1))
+    picks = list(order[:3]) + list(order[-3:]) + list(order[len(order) // 2: len(order) // 2 + 3])
+    for flat in picks:
+        h, i = divmod(int(flat), S // qblk)
+        wo, wlse = _oracle_block_rows(q, k, v, bi, bc, 0, h, i, qblk, S)
+        r = slice(i * qblk, (i + 1) * qblk)
+        assert_close_o(f32(o[0, h, r]), wo, "zipf q-block (%d,%d) count %d" % (h, i, counts[0, h, i]))
+        assert_close_stat(f32(lse[0, h, r]), wlse, "zipf lse")
+
+
+def test_cfg4_padded_threshold_pipeline(dev):
+    """N=32760 (padded to 32768), d=64, clustered keys: statistics -> vote mask -> index lists
+    -> sparse attention, two heads; each stage checked on sampled q-blocks."""
+    print("case cfg4 padded pipeline", flush=True)
+    B, H, S, D = 1, 2, 32760, 64
+    q, k, v = wl.clustered_qkv(B, H, S, D, seed=7)
+    qd, kd, vd = to_dev(dev, q, k, v)
+    Sp, SB = 32768, 256
+    mx = torch.empty((B, H, 1, Sp), device=dev)
+    dn = torch.empty((B, H, 1, Sp), device=dev)
+    capi.maxq_denom(mx, dn, qd, kd)
+    assert np.all(f32(mx)[..., S:] == 0) and np.all(np.isneginf(f32(dn)[..., S:]))
+    rng = np.random.default_rng(8)
+    blocks = [(int(rng.integers(H)), int(rng.integers(SB))) for _ in range(4)] + [(0, SB - 1)]   # incl. the ragged block
+    kf = f32(k)
+    for h, i in blocks:
+        r = slice(i * 128, min(S, (i + 1) * 128))
+        s = f32(q[0, h, r]) @ kf[0, h].T
+        m = s.max(1)
+        d = np.exp2((s - m[:, None]) * (orc.LOG2E / 8.0)).sum(1)
+        assert_close_stat(f32(mx)[0, h, 0, r], m, "max_q", atol=1e-3)
+        assert_close_stat(f32(dn)[0, h, 0, r], d, "denom")
+    # threshold: keep roughly 8 % of the (q-block, 64-key block) pairs of head 0, from sampled q-blocks
+    samp = []
+    for i in range(0, SB, 32):
+        r = slice(i * 128, min(S, (i + 1) * 128))
+        s = f32(q[0, 0, r]) @ kf[0, 0].T
+        p = np.exp2((s - f32(mx)[0, 0, 0, r, None]) * (orc.LOG2E / 8.0)) / f32(dn)[0, 0, 0, r, None]
+        pm = np.concatenate([p.max(0), np.zeros(Sp - S, np.float32)]).reshape(-1, 64).max(1)
+        samp.append(pm)
+    thr = float(np.quantile(np.concatenate(samp), 0.92))
+    mask = torch.zeros((B, H, SB, Sp), dtype=torch.int32, device=dev)
+    capi.booleanmask_128(mask, mx, dn, qd, kd, thr)
+    kvi = torch.full((B, H, SB, Sp), Sp, dtype=torch.int32, device=dev)
+    kvn = torch.zeros((B, H, SB), dtype=torch.int32, device=dev)
+    capi.booleanmask_to_indexmask(kvi, kvn, mask, S)
+    mh = mask.cpu().numpy()
+    assert mh.min() >= 0 and mh.max() <= 8 and np.all(mh[..., S:] == 0)
+    wi, wn = orc.booleanmask_to_indexmask(mh, S)                                   # bit-exact compaction
+    assert np.array_equal(kvn.cpu().numpy(), wn) and np.array_equal(kvi.cpu().numpy(), wi)
+    blockmask = orc.block_mask_from_votes(mh[:, :1], S)
+    assert 0.02 < blockmask.mean() < 0.3, blockmask.mean()
+    for h, i in blocks:
+        r = slice(i * 128, min(S, (i + 1) * 128))
+        s = f32(q[0, h, r]) @ kf[0, h].T
+        p = np.exp2((s - f32(mx)[0, h, 0, r, None]) * (orc.LOG2E / 8.0)) / f32(dn)[0, h, 0, r, None]
+        pmax = p.max(0)
+        near = np.abs(pmax - thr) <= 1e-2 * thr
+        assert np.array_equal((mh[0, h, i, :S] > 0) | near, (pmax > thr) | near), "mask row (%d,%d)" % (h, i)
+    o = torch.full_like(qd, float("nan"))
+    capi.sp_attn(o, qd, kd, vd, kvi, kvn)
+    assert torch.isfinite(o.float()).all()
+    vf = f32(v)
+    for h, i in blocks:
+        r = slice(i * 128, min(S, (i + 1) * 128))
+        lst = wi[0, h, i, : wn[0, h, i]]
+        s = f32(q[0, h, r]) @ kf[0, h, lst].T
+        pp, den, _ = orc._softmax_rows(s, 0.125, True)
+        assert_close_o(f32(o[0, h, r]), (pp @ vf[0, h, lst]) / den[:, None], "cfg4 sparse rows (%d,%d)" % (h, i))

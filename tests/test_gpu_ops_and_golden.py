@@ -1,0 +1,135 @@
+"""GPU: golden fixtures, the torch.ops.cuda_attn operator path and the functionals."""
+import glob
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from fgattn_tk_cuda_amd import capi, workloads as wl
+from oracle import spattn_oracle as orc
+from helpers import assert_close_o, assert_close_stat, f32, to_dev
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def _bf(x, dev):
+    return torch.from_numpy(np.ascontiguousarray(x)).to(torch.bfloat16).to(dev)
+
+
+@pytest.mark.parametrize("name", ["sparse_d64_q64", "sparse_d128_q128", "dense_d64"])
+def test_sp_attn_golden(dev, name):
+    print("case golden", name, flush=True)
+    g = np.load(os.path.join(GOLD, name + ".npz"))
+    q, k, v = (_bf(g[x][None, None], dev) for x in "qkv")
+    idx = torch.from_numpy(g["kv_indices"]).to(dev)
+    num = torch.from_numpy(g["kv_num_indices"]).to(dev)
+    o = torch.full_like(q, float("nan"))
+    lse = torch.full(q.shape[:3], float("nan"), device=dev)
+    capi.sp_attn(o, q, k, v, idx, num, lse=lse, qblk=int(g["qblk"]))
+    assert_close_o(f32(o)[0, 0], g["o"], name)
+    assert_close_stat(f32(lse)[0, 0], g["lse"], name + " lse")
+    if name == "dense_d64":
+        o2 = torch.full_like(q, float("nan"))
+        capi.full_attn(o2, q, k, v)
+        assert_close_o(f32(o2)[0, 0], g["o"], "full_attn golden")
+
+
+@pytest.mark.parametrize("name", ["prepass_d64", "prepass_d128"])
+def test_prepass_golden(dev, name):
+    print("case golden", name, flush=True)
+    g = np.load(os.path.join(GOLD, name + ".npz"))
+    q, k = (_bf(g[x][None, None], dev) for x in "qk")
+    S = q.shape[2]
+    Sp = orc.padded_len(S)
+    mx = torch.empty((1, 1, 1, Sp), device=dev)
+    dn = torch.empty((1, 1, 1, Sp), device=dev)
+    capi.maxq_denom(mx, dn, q, k)
+    assert_close_stat(f32(mx)[0, 0, 0, :S], g["max_q"], "max_q", atol=1e-4)
+    assert_close_stat(f32(dn)[0, 0, 0, :S], g["denom"], "denom")
+    mask = torch.zeros((1, 1, Sp // 128, Sp), dtype=torch.int32, device=dev)
+    capi.booleanmask_128(mask, mx, dn, q, k, float(g["thresh"]))
+    got = mask.cpu().numpy()
+    near = np.abs(g["pmax"] - g["thresh"]) <= 1e-2 * g["thresh"]
+    assert np.array_equal((got[..., :S] > 0) | near, (g["votes"][..., :S] > 0) | near)
+    gm = torch.from_numpy(g["votes"]).to(dev)
+    kvi = torch.full(gm.shape, Sp, dtype=torch.int32, device=dev)
+    kvn = torch.zeros(gm.shape[:3], dtype=torch.int32, device=dev)
+    capi.booleanmask_to_indexmask(kvi, kvn, gm, S)
+    assert np.array_equal(kvi.cpu().numpy(), g["kv_indices"]) and np.array_equal(kvn.cpu().numpy(), g["kv_num_indices"])
+
+
+def test_operator_extension_on_device(dev):
+    """The seven torch.ops.cuda_attn ops, used the way the reference's callers use them."""
+    print("case torch ops", flush=True)
+    import fgattn_tk_cuda_amd.spattn.cuda_attn  # noqa: F401
+    from fgattn_tk_cuda_amd.spattn import mask_utils as mu
+
+    ops = torch.ops.cuda_attn
+    B, H, S, D = 1, 2, 1000, 128
+    q, k, v = to_dev(dev, *wl.clustered_qkv(B, H, S, D, seed=71, sigma=0.5))
+    want = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float())
+    o = torch.empty_like(q)
+    ops.full_attn(o, q, k, v)
+    assert_close_o(f32(o), f32(want), "ops.full_attn")
+    Sp, SB = 1024, 8
+    kvi = torch.zeros((B, H, SB, Sp), dtype=torch.int32, device=dev)
+    kvn = torch.zeros((B, H, SB), dtype=torch.int32, device=dev)
+    ops.all_index_mask(kvi, kvn, B, H, SB, S)
+    o2 = torch.empty_like(q)
+    ops.sp_attn(o2, q, k, v, kvi, kvn)
+    assert_close_o(f32(o2), f32(want), "ops.sp_attn identity list")
+    # a list per 64 rows is recognised by the number of q-blocks
+    kvi64, kvn64 = to_dev(dev, *wl.permuted_all_index(B, H, S, qblk=64, seed=72))
+    ops.sp_attn(o2, q, k, v, kvi64, kvn64)
+    assert_close_o(f32(o2), f32(want), "ops.sp_attn 64-row lists")
+    mx = torch.empty((B, H, 1, Sp), device=dev)
+    dn = torch.empty((B, H, 1, Sp), device=dev)
+    o3 = torch.empty_like(q)
+    ops.fullattn_maxq_denom(o3, mx, dn, q, k, v)
+    assert_close_o(f32(o3), f32(want), "ops.fullattn_maxq_denom")
+    mx2, dn2 = torch.empty_like(mx), torch.empty_like(dn)
+    ops.maxq_denom(mx2, dn2, q, k)
+    assert_close_stat(f32(mx2), f32(mx), "max_q fused vs alone", atol=1e-4)
+    assert_close_stat(f32(dn2), f32(dn), "denom fused vs alone")
+    # the wrappers: torch definition of the mask vs the device path
+    thr = 0.02
+    dev_mask = mu.qk_bitmask_cuda(q, k, thr)[..., :S]
+    ref_mask = mu.qk_bitmask(q.float(), k.float(), thr)
+    _, pmax = orc.booleanmask_128(f32(mx2), f32(dn2), f32(q), f32(k), thr)
+    near = torch.from_numpy(np.abs(pmax - thr) <= 1e-2 * thr).to(dev)
+    assert torch.equal(dev_mask | near, ref_mask | near)
+    idx_d, num_d = mu.qk_indexmask_cuda(q, k, thr)
+    idx_r, num_r = mu.bitmask_to_indexmask(mu.qk_bitmask_cuda(q, k, thr))
+    assert torch.equal(idx_d, idx_r) and torch.equal(num_d, num_r)
+    # errors are raised, not swallowed
+    with pytest.raises(RuntimeError):
+        ops.full_attn(o, q.float(), k, v)
+    with pytest.raises(RuntimeError):
+        ops.sp_attn(o, q, k, v, kvi[:, :, :3].contiguous(), kvn)
+
+
+def test_functionals_with_mask_cache(dev):
+    print("case functionals", flush=True)
+    from fgattn_tk_cuda_amd.spattn import mask_utils as mu, sparseattn_functionals as fn
+
+    B, H, S, D = 1, 2, 900, 64
+    q, k, v = to_dev(dev, *wl.clustered_qkv(B, H, S, D, seed=81, sigma=0.7))
+    dense = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float())
+    assert_close_o(f32(fn.baseline_attn(q, k, v, 0, 0)), f32(dense), "baseline_attn")
+    assert_close_o(f32(fn.baseline_attn_maxq_denom(q, k, v, 0, 0)), f32(dense), "baseline_attn_maxq_denom")
+    for cache in (mu.NaiveMaskCache([0]), mu.BitMaskCache([0]), mu.CompressedBitMaskCache([0])):
+        f = fn.cached_attn_cuda if isinstance(cache, mu.NaiveMaskCache) else fn.bitmaskcached_attn_cuda
+        o0 = f(q, k, v, 7, 0, thresh=0.01, blocksz=128, mask_cache=cache)       # step 0: dense + cache fill
+        assert_close_o(f32(o0), f32(dense), "cache fill step")
+        o1 = f(q, k, v, 7, 1, thresh=0.01, blocksz=128, mask_cache=cache)       # step 1: sparse from cache
+        kvi, kvn = cache.get_mask_from_cache(7)
+        want, _ = orc.sp_attn(f32(q), f32(k), f32(v), kvi.cpu().numpy(), kvn.cpu().numpy(), qblk=128)
+        assert_close_o(f32(o1), want, "sparse step from %s" % type(cache).__name__)
+        assert 0 < kvn.float().mean().item() < S
+    o2 = fn.attn_computed_with_sparse_mask_cuda(q, k, v, thresh=0.01, blocksz=128)
+    assert_close_o(f32(o2), want, "attn_computed_with_sparse_mask_cuda")
+    o3 = fn.attn_2xmask_cuda(q, k, v, 0, 0, blocksz=128)
+    w3 = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float()[:, :, 0:2 * (S // 2):2], v.float()[:, :, 0:2 * (S // 2):2])
+    assert_close_o(f32(o3), f32(w3), "attn_2xmask_cuda")

@@ -1,0 +1,94 @@
+"""Host-side logic that needs no GPU: workload generators, the torch-level mask helpers
+and the operator registration."""
+import numpy as np
+import pytest
+import torch
+
+from fgattn_tk_cuda_amd import capi, workloads as wl
+from oracle import spattn_oracle as orc
+
+
+def test_uniform_block_lists():
+    B, H, S = 2, 3, 4096
+    idx, cnt = wl.uniform_block_lists(B, H, S, 64, 64, 6, seed=1)
+    assert idx.shape == (B, H, 64, 6) and idx.dtype == torch.int32 and torch.all(cnt == 6)
+    a = idx.numpy()
+    assert np.all(np.diff(a, axis=-1) > 0)                                  # sorted, unique
+    assert np.all((a == np.arange(64)[None, None, :, None]).any(-1))        # diagonal kept
+    idx2, _ = wl.uniform_block_lists(B, H, S, 64, 64, 6, seed=1)
+    assert torch.equal(idx, idx2)                                           # seeded
+    idx3, _ = wl.uniform_block_lists(1, 1, 1024, 128, 64, 4, seed=2)        # q-block 128: diagonal = block 2i
+    assert np.all((idx3.numpy()[0, 0] == 2 * np.arange(8)[:, None]).any(-1))
+
+
+def test_ragged_and_zipf_lists():
+    counts = wl.zipf_counts(1, 2, 32, s=1.2, lo=1, hi=16, seed=3)
+    assert counts.min() >= 1 and counts.max() <= 16
+    idx, cnt = wl.ragged_block_lists(1, 2, 2048, 64, 64, counts, seed=4)
+    assert np.array_equal(cnt.numpy(), counts)
+    for h in range(2):
+        for i in range(32):
+            c = int(cnt[0, h, i])
+            row = idx[0, h, i].numpy()
+            assert np.all(np.diff(row[:c]) > 0) and i in row[:c] and np.all(row[c:] == -1)
+
+
+def test_kept_block_flops_headline():
+    # 26 of 256 blocks per row, 256 rows per head, 2*32 heads
+    assert wl.kept_block_flops(2 * 32 * 256 * 26, 64, 64, 128) == pytest.approx(0.8934e12, rel=1e-3)
+
+
+def test_infer_qblk():
+    assert capi.infer_qblk(16384, 256) == 64 and capi.infer_qblk(16384, 128) == 128
+    assert capi.infer_qblk(32760, 256) == 128 and capi.infer_qblk(100, 1) == 128
+    with pytest.raises(ValueError):
+        capi.infer_qblk(16384, 100)
+
+
+def test_capi_rejects_host_tensors_without_touching_the_device():
+    q = torch.zeros((1, 1, 128, 64), dtype=torch.bfloat16)
+    with pytest.raises(ValueError):
+        capi.full_attn(torch.zeros_like(q), q, q, q)
+
+
+def test_torch_mask_helpers_match_oracle():
+    from fgattn_tk_cuda_amd.spattn import mask_utils as mu
+
+    rng = np.random.default_rng(5)
+    mask = (rng.random((2, 2, 3, 256)) < 0.2).astype(np.int32)
+    idx, cnt = mu.bitmask_to_indexmask(torch.from_numpy(mask))
+    wi, wn = orc.booleanmask_to_indexmask(mask, 256)
+    assert np.array_equal(idx.numpy(), wi) and np.array_equal(cnt.numpy(), wn)
+    q, k, _ = (t.float() for t in wl.clustered_qkv(1, 2, 300, 64, seed=6, sigma=0.7))
+    got = mu.qk_bitmask(q, k, thresh=0.02, blocksz=128).numpy()
+    mx, dn = orc.maxq_denom(q.numpy(), k.numpy())
+    votes, pmax = orc.booleanmask_128(mx, dn, q.numpy(), k.numpy(), 0.02)
+    near = np.abs(pmax - 0.02) <= 1e-3 * 0.02
+    assert np.array_equal(got | near, (votes[..., :300] > 0) | near)
+    b = torch.from_numpy(rng.random((2, 3, 64)) < 0.5)
+    assert torch.equal(mu.unpack(mu.pack(b)), b)
+    assert mu.pack(torch.tensor([[True, False, False, False, False, False, False, True]])).item() == 129
+    a = torch.rand(300, 8)
+    assert torch.equal(mu.attnmapor(a, 128)[2], a[256:].max(0).values)
+    assert torch.equal(mu.attnmapand(a, 128)[0], a[:128].min(0).values)
+    assert mu.attnmapbroadcast(torch.rand(2, 4), 128).shape == (256, 4)
+    cache = mu.NaiveMaskCache(compute_cache_at=[0, 5])
+    assert cache.run_fullattn(5) and not cache.run_fullattn(1)
+    cache.update_cache(3, "i", "n")
+    assert cache.get_mask_from_cache(3) == ("i", "n")
+
+
+def test_operator_extension_registers_the_seven_ops():
+    import fgattn_tk_cuda_amd.spattn.cuda_attn as ext
+
+    names = ["full_attn", "sp_attn", "all_index_mask", "maxq_denom", "booleanmask_128", "booleanmask_to_indexmask",
+             "fullattn_maxq_denom"]
+    for n in names:
+        assert hasattr(ext, n) and hasattr(torch.ops.cuda_attn, n)
+    # Meta kernels let fake tensors trace through the ops (python/extension.cpp:74-79)
+    q = torch.zeros((1, 2, 256, 128), dtype=torch.bfloat16, device="meta")
+    torch.ops.cuda_attn.full_attn(q, q, q, q)
+    idx = torch.zeros((1, 2, 2, 256), dtype=torch.int32, device="meta")
+    torch.ops.cuda_attn.sp_attn(q, q, q, q, idx, idx)
+    schema = str(torch.ops.cuda_attn.sp_attn.default._schema)
+    assert "Tensor(a!) o" in schema and "kv_num_indices" in schema

@@ -1,0 +1,206 @@
+"""Pins the CPU oracle: golden fixtures (independent fp64 loops), library routines that
+special cases reduce to, invariants, and brute force.  Runs without a GPU."""
+import glob
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from fgattn_tk_cuda_amd import workloads as wl
+from oracle import cpu_masked_attention as cma
+from oracle import spattn_oracle as orc
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def _qkv(B, H, S, D, seed):
+    return tuple(t.float().numpy() for t in wl.randn_qkv(B, H, S, D, seed=seed))
+
+
+def test_fixture_files_present():
+    names = sorted(os.path.basename(p) for p in glob.glob(os.path.join(GOLD, "*.npz")))
+    assert names == ["dense_d64.npz", "prepass_d128.npz", "prepass_d64.npz", "sparse_d128_q128.npz", "sparse_d64_q64.npz"]
+
+
+@pytest.mark.parametrize("name", ["sparse_d64_q64", "sparse_d128_q128", "dense_d64"])
+def test_sp_attn_matches_golden(name):
+    g = np.load(os.path.join(GOLD, name + ".npz"))
+    q, k, v = (g[x][None, None] for x in "qkv")
+    o, lse = orc.sp_attn(q, k, v, g["kv_indices"], g["kv_num_indices"], qblk=int(g["qblk"]), round_p=False)
+    assert np.allclose(o[0, 0], g["o"], atol=2e-5, rtol=1e-4)
+    assert np.allclose(lse[0, 0], g["lse"], atol=1e-4, rtol=1e-5)
+    # with P rounded to bf16 (what the kernels do) the result stays well inside the contract
+    o2, _ = orc.sp_attn(q, k, v, g["kv_indices"], g["kv_num_indices"], qblk=int(g["qblk"]), round_p=True)
+    assert np.abs(o2[0, 0] - g["o"]).max() < 5e-3
+
+
+def test_full_attn_matches_golden_and_sdpa():
+    g = np.load(os.path.join(GOLD, "dense_d64.npz"))
+    q, k, v = (g[x][None, None] for x in "qkv")
+    o, mx, dn = orc.full_attn(q, k, v, round_p=False)
+    assert np.allclose(o[0, 0], g["o"], atol=2e-5, rtol=1e-4)
+    q, k, v = _qkv(2, 2, 300, 64, 1)
+    o, _, _ = orc.full_attn(q, k, v, round_p=False)
+    want = torch.nn.functional.scaled_dot_product_attention(*(torch.from_numpy(x) for x in (q, k, v))).numpy()
+    assert np.allclose(o, want, atol=2e-5, rtol=1e-4)
+    o, _, _ = orc.full_attn(q, k, v, kv_len=250, round_p=False)
+    want = torch.nn.functional.scaled_dot_product_attention(torch.from_numpy(q), torch.from_numpy(k[:, :, :250]), torch.from_numpy(v[:, :, :250])).numpy()
+    assert np.allclose(o, want, atol=2e-5, rtol=1e-4)
+
+
+@pytest.mark.parametrize("qblk", [64, 128])
+def test_sp_attn_permuted_full_list_is_sdpa(qblk):
+    """The reference's own sparse test: a permutation of all keys (python/test/test_extension.py:61-89)."""
+    B, H, S, D = 1, 2, 333, 64
+    q, k, v = _qkv(B, H, S, D, 2)
+    idx, num = wl.permuted_all_index(B, H, S, qblk=qblk, seed=3)
+    o, lse = orc.sp_attn(q, k, v, idx.numpy(), num.numpy(), qblk=qblk, round_p=False)
+    tq, tk, tv = (torch.from_numpy(x) for x in (q, k, v))
+    want = torch.nn.functional.scaled_dot_product_attention(tq, tk, tv).numpy()
+    assert np.allclose(o, want, atol=2e-5, rtol=1e-4)
+    s = torch.einsum("bhmd,bhnd->bhmn", tq, tk) / math.sqrt(D)
+    assert np.allclose(lse, torch.logsumexp(s, -1).numpy(), atol=1e-4)
+
+
+def test_sp_attn_invariants():
+    B, H, S, D = 1, 1, 256, 64
+    q, k, v = _qkv(B, H, S, D, 4)
+    rng = np.random.default_rng(5)
+    ms = 256
+    base = np.full((B, H, 2, ms), ms, np.int32)
+    base[0, 0, 0, :100] = rng.permutation(S)[:100]
+    base[0, 0, 1, :37] = rng.permutation(S)[:37]
+    num = np.array([[[100, 37]]], np.int32)
+    o0, l0 = orc.sp_attn(q, k, v, base, num, round_p=False)
+    perm = base.copy()
+    perm[0, 0, 0, :100] = perm[0, 0, 0, rng.permutation(100)]
+    o1, _ = orc.sp_attn(q, k, v, perm, num, round_p=False)
+    assert np.allclose(o0, o1, atol=1e-5)                       # order does not matter
+    dup = base.copy()
+    dup[0, 0, 0, 100:200] = base[0, 0, 0, :100]
+    dup[0, 0, 1, 37:74] = base[0, 0, 1, :37]
+    o2, l2 = orc.sp_attn(q, k, v, dup, num * 2, round_p=False)
+    assert np.allclose(o0, o2, atol=1e-5)                       # a duplicated list changes nothing ...
+    assert np.allclose(l2, l0 + math.log(2), atol=1e-5)         # ... but the log-sum-exp by log 2
+    one = np.full((B, H, 2, ms), ms, np.int32)
+    one[0, 0, :, 0] = [17, 200]
+    o3, _ = orc.sp_attn(q, k, v, one, np.ones((B, H, 2), np.int32))
+    assert np.array_equal(o3[0, 0, :128], np.repeat(v[0, 0, 17:18], 128, 0))   # a single key returns its V row
+    assert np.array_equal(o3[0, 0, 128:], np.repeat(v[0, 0, 200:201], 128, 0))
+    # entries past the count and entries >= S are ignored; an empty list gives zeros / -inf
+    bad = base.copy()
+    bad[0, 0, 0, 100:110] = 3
+    bad[0, 0, 1, 5] = 9999
+    num2 = np.array([[[100, 37]]], np.int32)
+    o4, _ = orc.sp_attn(q, k, v, bad, num2, round_p=False)
+    keep = [c for j, c in enumerate(base[0, 0, 1, :37]) if j != 5]
+    ref = base.copy()
+    ref[0, 0, 1, :36] = keep
+    o5, _ = orc.sp_attn(q, k, v, ref, np.array([[[100, 36]]], np.int32), round_p=False)
+    assert np.allclose(o4, o5, atol=1e-6)
+    o6, l6 = orc.sp_attn(q, k, v, base, np.zeros((B, H, 2), np.int32))
+    assert np.all(o6 == 0) and np.all(np.isneginf(l6))
+
+
+def test_block_lists_expand_to_token_lists():
+    B, H, S = 1, 2, 1000
+    bi, bc = wl.ragged_block_lists(B, H, S, 64, 64, np.array([[3] * 16, [16] * 16]), seed=6)
+    tok, num = orc.block_list_to_token_list(bi.numpy(), bc.numpy(), S)
+    tok2, num2 = wl.blocks_to_tokens(bi, bc, S)
+    assert np.array_equal(tok, tok2.numpy()) and np.array_equal(num, num2.numpy())
+    for h in range(H):
+        for i in range(16):
+            want = sorted(t for j in bi[0, h, i, : bc[0, h, i]].tolist() for t in range(64 * j, min(S, 64 * j + 64)))
+            assert tok[0, h, i, : num[0, h, i]].tolist() == want
+
+
+def test_cpu_baseline_matches_oracle():
+    B, H, S, D, qblk = 1, 1, 512, 64, 64
+    q, k, v = wl.randn_qkv(B, H, S, D, seed=7, dtype=torch.float32)
+    bi, bc = wl.uniform_block_lists(B, H, S, qblk, 64, 3, seed=8)
+    got = cma.masked_attention_rows(q[0, 0], k[0, 0], v[0, 0], bi[0, 0], bc[0, 0], 64, 320, qblk, 64).numpy()
+    tok, num = wl.blocks_to_tokens(bi, bc, S)
+    want, _ = orc.sp_attn(q.numpy(), k.numpy(), v.numpy(), tok.numpy(), num.numpy(), qblk=qblk, round_p=False)
+    assert np.allclose(got, want[0, 0, 64:320], atol=2e-5, rtol=1e-4)
+
+
+@pytest.mark.parametrize("name", ["prepass_d64", "prepass_d128"])
+def test_prepass_matches_golden(name):
+    g = np.load(os.path.join(GOLD, name + ".npz"))
+    q, k = g["q"][None, None], g["k"][None, None]
+    S = q.shape[2]
+    mx, dn = orc.maxq_denom(q, k)
+    assert np.allclose(mx[0, 0, 0, :S], g["max_q"], rtol=1e-5, atol=1e-4)
+    assert np.allclose(dn[0, 0, 0, :S], g["denom"], rtol=1e-4)
+    assert np.all(mx[..., S:] == 0) and np.all(np.isneginf(dn[..., S:]))      # pad rows
+    votes, pmax = orc.booleanmask_128(mx, dn, q, k, float(g["thresh"]))
+    assert np.allclose(pmax, g["pmax"], rtol=1e-3, atol=1e-9)
+    near = np.abs(g["pmax"] - g["thresh"]) <= 1e-3 * g["thresh"]
+    assert np.array_equal((votes[..., :S] > 0) | near, (g["votes"][..., :S] > 0) | near)
+    assert (votes == g["votes"]).mean() > 0.999
+    idx, num = orc.booleanmask_to_indexmask(g["votes"], S)
+    assert np.array_equal(idx, g["kv_indices"]) and np.array_equal(num, g["kv_num_indices"])
+
+
+def test_maxq_denom_closed_forms():
+    """The reference's own check (python/test/spattn/test_mask_utils.py:33-56)."""
+    B, H, S, D = 1, 2, 300, 128
+    q, k, _ = _qkv(B, H, S, D, 9)
+    mx, dn = orc.maxq_denom(q, k)
+    for h in range(H):
+        s = torch.from_numpy(q[0, h]) @ torch.from_numpy(k[0, h]).T
+        assert np.allclose(mx[0, h, 0, :S], s.max(-1).values.numpy(), atol=1e-4)
+        d = torch.exp((s - s.max(-1, keepdim=True).values) / math.sqrt(D)).sum(-1)
+        assert np.allclose(dn[0, h, 0, :S], d.numpy(), rtol=1e-4)
+    mx2, dn2 = orc.maxq_denom(q, k, kv_len=200)
+    s = torch.from_numpy(q[0, 0]) @ torch.from_numpy(k[0, 0, :200]).T
+    assert np.allclose(mx2[0, 0, 0, :S], s.max(-1).values.numpy(), atol=1e-4)
+
+
+def test_booleanmask_is_maxpooled_threshold():
+    """>0 of the vote mask is the 128-row max-pool of softmax > thresh
+    (python/spattn/mask_utils.py:126-142,206-222), here with torch's softmax and max_pool."""
+    B, H, S, D = 1, 2, 300, 64
+    q, k, _ = (t.float() for t in wl.clustered_qkv(B, H, S, D, seed=10, sigma=0.7))
+    mx, dn = orc.maxq_denom(q.numpy(), k.numpy())
+    thr = 0.02
+    votes, pmax = orc.booleanmask_128(mx, dn, q.numpy(), k.numpy(), thr)
+    for h in range(H):
+        p = torch.softmax(q[0, h] @ k[0, h].T / math.sqrt(D), -1)
+        hit = (p > thr).float()[None]
+        pooled = torch.nn.functional.max_pool2d(torch.nn.functional.pad(hit, (0, 0, 0, (-S) % 128)), (128, 1))[0] > 0
+        near = np.abs(pmax[0, h] - thr) <= 1e-3 * thr
+        assert np.array_equal((votes[0, h, :, :S] > 0) | near, pooled.numpy() | near)
+        # vote count = number of 16-row groups that hit
+        cnt = torch.nn.functional.max_pool2d(torch.nn.functional.pad(hit, (0, 0, 0, (-S) % 16)), (16, 1))[0]
+        cnt = torch.nn.functional.pad(cnt, (0, 0, 0, (-cnt.shape[0]) % 8)).view(-1, 8, S).sum(1)
+        assert ((votes[0, h, :, :S] == cnt.numpy()) | near).all()
+    assert np.all(votes[..., S:] == 0)
+
+
+def test_booleanmask_to_indexmask_exact():
+    rng = np.random.default_rng(11)
+    mask = (rng.random((2, 2, 3, 256)) < 0.2) * rng.integers(1, 9, (2, 2, 3, 256))
+    idx, num = orc.booleanmask_to_indexmask(mask, 200)
+    for b in range(2):
+        for h in range(2):
+            for i in range(3):
+                kept = [c for c in range(200) if mask[b, h, i, c] > 0]       # plain loop
+                assert num[b, h, i] == len(kept)
+                assert idx[b, h, i, : len(kept)].tolist() == kept
+                assert np.all(idx[b, h, i, len(kept):] == 256)
+    idx2, num2 = orc.booleanmask_to_indexmask(np.zeros((1, 1, 1, 128), np.int32), 128)
+    assert num2[0, 0, 0] == 0 and np.all(idx2 == 128)
+
+
+def test_all_index_mask():
+    idx, num = orc.all_index_mask(1, 2, 3, 300, 384)
+    assert idx.shape == (1, 2, 3, 384) and np.all(idx == np.arange(384)) and np.all(num == 300)
+
+
+def test_bf16_round():
+    x = np.array([1.0, 1.00390625, 1.01171875, -3.1415926, 1e-30, 65504.0], np.float32)
+    want = torch.from_numpy(x).to(torch.bfloat16).float().numpy()
+    assert np.array_equal(orc.bf16_round(x), want)
