@@ -31,6 +31,13 @@ from fgattn_tk_cuda_amd import capi, workloads as wl  # noqa: E402
 PEAK_BF16_TFLOPS = 2500.0
 PEAK_HBM_GBPS = 8000.0
 
+# HBM-side bytes per launch from `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs of this
+# file (--only sparse / --only compact), scaled by what the same counters read for the plain
+# 1 GiB copy of --only copy (FETCH_SIZE x2.0, WRITE_SIZE x1.0).  Text summaries of those runs
+# sit in profiles/counters_*.txt; they are measured offline, not in this process.
+TRAFFIC_SPARSE_BYTES = 5.36e9 + 0.675e9     # fetch + write of attn_fwd_kernel<128,64,KV_BLOCKS>
+TRAFFIC_COMPACT_BYTES = 805.4e6 + 64.5e6    # fetch + write of compact_kernel
+
 
 def time_steps(fn, steps: int, warmup: int):
     """Average milliseconds of fn() over `steps` launches, HIP events on the launch stream."""
@@ -94,6 +101,16 @@ def bench_compaction(dev, steps, warmup, seed=0):
     return dict(ms=ms, bytes=nbytes, kept=kept, shape=[B, H, SB, ms_])
 
 
+def bench_copy(dev, steps, warmup, seed=0):
+    """A plain 1 GiB device-to-device copy: the known-size kernel that the FETCH_SIZE /
+    WRITE_SIZE counters of the other kernels are scaled by."""
+    n = 1 << 28
+    a = torch.ones((n,), dtype=torch.float32, device=dev)
+    b = torch.empty_like(a)
+    ms, _ = time_steps(lambda: b.copy_(a), steps, warmup)
+    return dict(ms=ms, read_bytes=4.0 * n, write_bytes=4.0 * n)
+
+
 def bench_dense(dev, steps, warmup, seed=0):
     c = wl.CONFIGS["cfg2_dense"]
     B, H, S, D = c["B"], c["H"], c["S"], c["D"]
@@ -118,32 +135,41 @@ def bench_sweeps(dev, steps, warmup, seed=0, heads=None):
     return dict(ms_maxq_denom=ms1, ms_booleanmask=ms2, flops=flops, mask_bytes=4.0 * mask.numel())
 
 
-def cpu_baseline(res, budget_s=20.0):
+def cpu_baseline(res, budget_s=15.0):
     """Dense-masked PyTorch attention on the host cores over a bounded sample of the
-    headline workload: whole q-blocks of head (0,0), as many as fit the time budget."""
+    headline workload: 2048-row slabs of successive heads until the time budget is used."""
     from oracle import cpu_masked_attention as cma
 
     q, k, v, bi, bc, _ = res["tensors"]
-    S, D, qblk, kvblk = res["S"], res["D"], res["qblk"], res["kvblk"]
-    qh, kh, vh = (t[0, 0].float().cpu() for t in (q, k, v))
-    bih, bch = bi[0, 0].cpu(), bc[0, 0].cpu()
+    B, H, S, D, qblk, kvblk = res["B"], res["H"], res["S"], res["D"], res["qblk"], res["kvblk"]
     cores = os.cpu_count() or 1
     torch.set_num_threads(cores)
     chunk = 2048
-    done_rows, kept, t_used = 0, 0, 0.0
-    while done_rows < S and t_used < budget_s:
-        r0, r1 = done_rows, min(S, done_rows + chunk)
-        t0 = time.perf_counter()
-        cma.masked_attention_rows(qh, kh, vh, bih, bch, r0, r1, qblk, kvblk)
-        t_used += time.perf_counter() - t0
-        kept += int(bch[r0 // qblk: wl.ceil_div(r1, qblk)].sum())
-        done_rows = r1
+    rows, kept, t_used, heads = 0, 0, 0.0, 0
+    for bh in range(B * H):
+        if t_used >= budget_s:
+            break
+        b, h = divmod(bh, H)
+        qh, kh, vh = (t[b, h].float().cpu() for t in (q, k, v))
+        bih, bch = bi[b, h].cpu(), bc[b, h].cpu()
+        heads += 1
+        for r0 in range(0, S, chunk):
+            r1 = min(S, r0 + chunk)
+            t0 = time.perf_counter()
+            cma.masked_attention_rows(qh, kh, vh, bih, bch, r0, r1, qblk, kvblk)
+            t_used += time.perf_counter() - t0
+            kept += int(bch[r0 // qblk: wl.ceil_div(r1, qblk)].sum())
+            rows += r1 - r0
+            if t_used >= budget_s:
+                break
     flops = wl.kept_block_flops(kept, qblk, kvblk, D)
     return {
         "value": flops / t_used / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
-        "sample": "dense-masked fp32 torch attention (QK^T, -inf outside kept blocks, softmax, PV) on %d of %d query "
-                  "rows of head (0,0), %.1f s; kept-block flops of those rows / time" % (done_rows, S, t_used),
+        "sample": "dense-masked fp32 torch attention (QK^T, -inf outside kept blocks, softmax, PV) on %d query rows "
+                  "(%d heads touched) of the %d in the workload, %.1f s; kept-block flops of those rows / time"
+                  % (rows, heads, B * H * S, t_used),
         "seconds": t_used,
+        "ms_per_step_extrapolated": t_used * (B * H * S / max(rows, 1)) * 1e3,
     }
 
 
@@ -154,7 +180,7 @@ def main(argv=None) -> int:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-extras", action="store_true", help="only the headline kernel")
-    ap.add_argument("--only", default="", help="run one leg only: sparse|compact|dense|sweeps (no JSON contract)")
+    ap.add_argument("--only", default="", help="run one leg only: sparse|compact|dense|sweeps|copy (no JSON contract)")
     args = ap.parse_args(argv)
     if args.gpus != 1:
         print("bench.py: this library is single-GPU; run with --gpus 1 (got %d)" % args.gpus, file=sys.stderr)
@@ -167,7 +193,8 @@ def main(argv=None) -> int:
     torch.cuda.set_device(dev)
 
     if args.only:
-        fn = {"sparse": bench_sparse, "compact": bench_compaction, "dense": bench_dense, "sweeps": bench_sweeps}[args.only]
+        fn = {"sparse": bench_sparse, "compact": bench_compaction, "dense": bench_dense, "sweeps": bench_sweeps,
+              "copy": bench_copy}[args.only]
         r = fn(dev, args.steps, args.warmup)
         r.pop("tensors", None)
         print(json.dumps(r))
@@ -184,7 +211,7 @@ def main(argv=None) -> int:
                                "26 of 256 key blocks per row incl. diagonal, bf16 O + fp32 lse",
                    "kept_blocks": res["kept_blocks"], "flops_per_step": res["flops"]},
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": None,
+                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_SPARSE_BYTES, "traffic_unit": "bytes",
                      "kernel": "attn_fwd_kernel<128,64,KV_BLOCKS>"},
     }
     if not args.no_extras:
@@ -193,7 +220,8 @@ def main(argv=None) -> int:
         out["mask_pass"] = {"kernel": "compact_kernel (booleanmask_to_indexmask)", "workload": "cfg4 mask %s int32, %.1f%% kept"
                             % (cp["shape"], 100.0 * cp["kept"] / np.prod(cp["shape"])), "ms": cp["ms"],
                             "roofline": {"bound": "hbm", "achieved": gbps, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                                         "frac": gbps / PEAK_HBM_GBPS, "traffic": None}}
+                                         "frac": gbps / PEAK_HBM_GBPS, "traffic": TRAFFIC_COMPACT_BYTES,
+                                         "traffic_unit": "bytes", "algorithmic_bytes": cp["bytes"]}}
         dn = bench_dense(dev, args.steps, args.warmup)
         out["dense_full_attn"] = {"workload": "cfg2: B=4 H=16 N=4096 d=64", "ms": dn["ms"],
                                   "tflops": dn["flops"] / (dn["ms"] * 1e-3) / 1e12,
