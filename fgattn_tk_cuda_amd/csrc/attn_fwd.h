@@ -140,25 +140,36 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   // ---- loader role: load i of a tile covers rows RPL*(4i + wave) .. +RPL-1 ----------
   const int ld_sub = lane / CPR;       // row within the load
   const int ld_slot = lane % CPR;      // 16-byte position within the row in LDS
-  // Row r of a tile stores its 16-byte chunk c at position c ^ swz(r).  Eight consecutive
-  // rows put one chunk into eight different 16-byte bank groups (the K reads), four
-  // consecutive rows put one 32-byte window into four different windows (the transposing
-  // V reads), and rows r and r+8 share a swizzle.
-  auto swz = [](int r) -> int { return D == 128 ? ((r & 7) << 1) : (((r & 3) << 1) | ((r >> 2) & 1)); };
+  // Row r of a tile stores its 16-byte chunk c at position c ^ swz(r).  The swizzle has a
+  // period of 16 rows and is chosen so that (K reads, ds_read_b128) one chunk of 16
+  // consecutive rows covers all sixteen 16-byte bank groups, and (transposing V reads) the
+  // two 32-byte windows that a read takes from each of four consecutive rows cover all
+  // eight 32-byte windows: both reads then run at the full LDS rate (measured: twice,
+  // resp. 1.45 times, the rate of a swizzle that only separates 8 rows).
+  auto swz = [](int r) -> int {
+    return D == 128 ? (((r & 3) << 2) | ((r >> 2) & 3)) : ((((r >> 1) & 1) << 2) | ((r >> 2) & 3));
+  };
   auto ld_row = [&](int i) -> int { return RPL * (4 * i + wave) + ld_sub; };
   auto ld_off = [&](int i) -> int { return (ld_slot ^ swz(ld_row(i))) << 4; };   // chunk offset within the row
   uint32_t ld_go[LPT];                 // lane offset within a contiguous 64-row tile
 #pragma unroll
   for (int i = 0; i < LPT; ++i) ld_go[i] = ld_row(i) * ROWB + ld_off(i);
 
-  // First key row of tile t (dense / block lists); kv_len marks "no such block".
-  auto tile_row0 = [&](int t) -> int {
-    if constexpr (MODE == KV_DENSE) return t * 64;
-    if constexpr (MODE == KV_BLOCKS) {
-      const int blk = lst[t];
-      return (blk >= 0 && blk <= (last_row >> 6)) ? blk * 64 : p.kv_len;
-    }
+  // First key row of a tile (dense / block lists) from its id; kv_len marks "no such block".
+  // The id of tile t is t itself (dense) or the t-th list entry (block lists).
+  auto tile_id = [&](int t) -> int {
+    if constexpr (MODE == KV_BLOCKS) return lst[t];
+    return t;
+  };
+  auto id_row0 = [&](int blk) -> int {
+    if constexpr (MODE == KV_DENSE) return blk * 64;
+    if constexpr (MODE == KV_BLOCKS) return (blk >= 0 && blk <= (last_row >> 6)) ? blk * 64 : p.kv_len;
     return 0;
+  };
+  // Same, for a tile that may lie past the end of the list (prefetched ids that are never used).
+  auto tile_id_clamped = [&](int t) -> int {
+    if constexpr (MODE == KV_BLOCKS) return lst[t < p.idx_stride ? t : p.idx_stride - 1];
+    return t;
   };
 
   // Token lists: the RPL token ids behind one load are wave-uniform, so they are fetched
@@ -203,7 +214,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     uint32_t lds;
     uint32_t go[LPT];
   };
-  auto prepare_tile = [&](int t, int slot, bool is_v) -> TileLoad {
+  auto prepare_tile = [&](int t, int id, int slot, bool is_v) -> TileLoad {
     TileLoad tl;
     tl.lds = smem_base + (uint32_t)slot * TILE + wave * 1024;
     const unsigned char* src = is_v ? vh : kh;
@@ -229,7 +240,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
         tok_fetch(t + 2);
       }
     } else {
-      const int r0 = tile_row0(t);
+      const int r0 = id_row0(id);
       if (r0 + 64 <= p.kv_len) {
         tl.base = src + (size_t)r0 * ROWB;   // whole tile in range
 #pragma unroll
@@ -249,7 +260,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   };
   auto load_part = [&](const TileLoad& tl, int i) { dma16(tl.base, tl.go[i], tl.lds + i * 4096); };
   auto issue_tile = [&](int t, int slot, bool is_v) {
-    const TileLoad tl = prepare_tile(t, slot, is_v);
+    const TileLoad tl = prepare_tile(t, tile_id(t), slot, is_v);
 #pragma unroll
     for (int i = 0; i < LPT; ++i) load_part(tl, i);
   };
@@ -282,23 +293,23 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   const int qrow = q0 + ln;
   const bool qrow_ok = qrow < p.S;
 
+  tok_fetch(0);
+  tok_resolve(0);
+  tok_fetch(1);
+  issue_phase(0);
+  // The Q loads are the only compiler-visible vector loads of the kernel.  They go out
+  // between the first copies so that their latency overlaps that of tile 0, and must have
+  // retired before the first counted wait.
   u32x4 qf[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     const u32x4 z = {0, 0, 0, 0};
     qf[t] = qrow_ok ? *reinterpret_cast<const u32x4*>(qh + (size_t)qrow * D + 16 * t + 8 * g) : z;
   }
-  // The Q loads must have retired before the first counted wait; they are the only
-  // compiler-visible vector loads of the kernel.
-#pragma unroll
-  for (int t = 0; t < NT; ++t) asm volatile("" ::"v"(qf[t]));
-
-  tok_fetch(0);
-  tok_resolve(0);
-  tok_fetch(1);
-  issue_phase(0);
   issue_phase(1);
   issue_phase(2);
+#pragma unroll
+  for (int t = 0; t < NT; ++t) asm volatile("" ::"v"(qf[t]));
 
   // Softmax state of this lane's query row.  Exponents are taken against a reference
   // mr_sf (in log2 units, = raw max * sf at the time it was set) that is only moved when
@@ -329,21 +340,24 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   // Transposing V read: in each 16-lane group, lane i addresses 4 dims of key (i>>2);
   // lane j receives dim j of those 4 keys.  Keys 4g..4g+3 (+8 for the second read) of
   // each 16-key step, dims 32db + 16*dhalf + 4*(i&3)..+3.
-  lds_cptr v_lo[HAS_V ? NDB : 1];
+  lds_cptr v_lo[HAS_V ? NDB : 1];    // keys 4g..4g+3 of a step
+  lds_cptr v_lo2[HAS_V ? NDB : 1];   // keys 8+4g..8+4g+3 of a step (their rows have another swizzle)
   if constexpr (HAS_V) {
     const int i16 = lane & 15;
     const int dhalf = (lane >> 4) & 1;
     const int r1 = ksub * KW + 4 * g + (i16 >> 2);
-    const int sw = swz(r1);   // also the swizzle of row r1 + 8, the second read
     const int cb = 2 * dhalf + ((i16 & 3) >> 1);
 #pragma unroll
-    for (int db = 0; db < NDB; ++db) v_lo[db] = smem_l + r1 * ROWB + (((4 * db + cb) ^ sw) << 4) + ((i16 & 1) << 3);
+    for (int db = 0; db < NDB; ++db) {
+      v_lo[db] = smem_l + r1 * ROWB + (((4 * db + cb) ^ swz(r1)) << 4) + ((i16 & 1) << 3);
+      v_lo2[db] = smem_l + (r1 + 8) * ROWB + (((4 * db + cb) ^ swz(r1 + 8)) << 4) + ((i16 & 1) << 3);
+    }
   }
 
   // ---- building blocks --------------------------------------------------------------
   // Keys of tile `it` that do not exist get -inf.  Accumulator register 4j+i of block mb
   // is key ksub*KW + 32mb + 8j + 4g + i of the tile.
-  auto mask_tile = [&](int it, f32x16 (&s)[NMB]) {
+  auto mask_tile = [&](int it, int id, f32x16 (&s)[NMB]) {
     if constexpr (MODE == KV_TOKENS) {
       const float* bias = reinterpret_cast<const float*>(smem + Cfg::kTotal - Cfg::kBiasBytes) + (it % Cfg::kBiasRing) * 64;
 #pragma unroll
@@ -357,7 +371,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
           s[mb][4 * j + 3] += bv.w;
         }
     } else {
-      const int r0 = tile_row0(it);
+      const int r0 = id_row0(id);
       if (r0 + 64 > p.kv_len) {
 #pragma unroll
         for (int mb = 0; mb < NMB; ++mb)
@@ -474,8 +488,9 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
 #pragma unroll
           for (int db = 0; db < NDB; ++db) {
             const lds_cptr a1 = v_lo[db] + vofs + (2 * mb + h) * 16 * ROWB;
+            const lds_cptr a2 = v_lo2[db] + vofs + (2 * mb + h) * 16 * ROWB;
             va[h][db][0] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((SPATTN_LDS s16x4*)a1));
-            va[h][db][1] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((SPATTN_LDS s16x4*)(a1 + 8 * ROWB)));
+            va[h][db][1] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((SPATTN_LDS s16x4*)a2));
           }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -498,7 +513,10 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   // it (scores in s_a), then V phase of tile it (ring slot VS) with the row maxima of tile
   // it+1 (scores in s_b).  In the steady state every later phase exists, so waits and
   // issues are unconditional.
-  auto tile_body = [&](auto ks_c, auto vs_c, auto steady_c, int it, f32x16 (&s_a)[NMB], f32x16 (&s_b)[NMB]) {
+  // id_v / id_k: ids of tiles it+1 and it+3 (it+4 without V), fetched ahead of time by the
+  // steady loop so that no list load sits between a barrier and the copies behind it;
+  // the generic form looks them up itself.
+  auto tile_body = [&](auto ks_c, auto vs_c, auto steady_c, int it, f32x16 (&s_a)[NMB], f32x16 (&s_b)[NMB], int id_v, int id_k) {
     constexpr int KS = decltype(ks_c)::value;
     constexpr int VS = decltype(vs_c)::value;
     constexpr bool STEADY = decltype(steady_c)::value;
@@ -508,7 +526,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
       __syncthreads();
       // phase j+3 is V(it+1) (with V) or K(it+4)
       if constexpr (STEADY) {
-        const TileLoad tl = HAS_V ? prepare_tile(it + 1, (VS + 2) & 3, true) : prepare_tile(it + 4, (KS + 3) & 3, false);
+        const TileLoad tl = HAS_V ? prepare_tile(it + 1, id_v, (VS + 2) & 3, true) : prepare_tile(it + 4, id_k, (KS + 3) & 3, false);
         qk_tile(std::true_type{}, KS * TILE, s_b, s_a, &tl);
       } else {
         if constexpr (HAS_V) {
@@ -518,7 +536,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
         }
         qk_tile(std::true_type{}, KS * TILE, s_b, s_a, nullptr);
       }
-      mask_tile(it + 1, s_b);
+      mask_tile(it + 1, STEADY ? id_v : tile_id(it + 1), s_b);
     }
     if constexpr (HAS_V) {
       const int j = 2 * it + 2;
@@ -526,7 +544,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
       __syncthreads();
       // phase j+3 is K(it+3)
       if constexpr (STEADY) {
-        const TileLoad tl = prepare_tile(it + 3, KS, false);
+        const TileLoad tl = prepare_tile(it + 3, id_k, KS, false);
         pv_tile(VS * TILE, &tl);
       } else {
         if (it + 3 < ntiles) issue_tile(it + 3, KS, false);
@@ -547,19 +565,31 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     __syncthreads();
     issue_phase(3);
     qk_tile(std::false_type{}, 0, s_e, s_e, nullptr);
-    mask_tile(0, s_e);
+    mask_tile(0, tile_id(0), s_e);
     maybe_rescale(row_stats(s_e));
 
     int it = 0;
     if constexpr (HAS_V) {
       // tile `it` has its next K tile in slot (2it+1)&3 and its V tile in slot (2it+2)&3
+      // w1..w3: ids of tiles it+1..it+3; two more are fetched per round, a round ahead
+      int w1 = 0, w2 = 0, w3 = 0;
+      if (4 < ntiles) {
+        w1 = tile_id(1);
+        w2 = tile_id(2);
+        w3 = tile_id(3);
+      }
       for (; it + 4 < ntiles; it += 2) {
-        tile_body(I1{}, I2{}, std::true_type{}, it, s_e, s_o);
-        tile_body(I3{}, I0{}, std::true_type{}, it + 1, s_o, s_e);
+        const int w4 = tile_id(it + 4);
+        const int w5 = tile_id_clamped(it + 5);
+        tile_body(I1{}, I2{}, std::true_type{}, it, s_e, s_o, w1, w3);
+        tile_body(I3{}, I0{}, std::true_type{}, it + 1, s_o, s_e, w2, w4);
+        w1 = w3;
+        w2 = w4;
+        w3 = w5;
       }
       for (; it + 1 < ntiles; ++it) {
-        if (it & 1) tile_body(I3{}, I0{}, std::false_type{}, it, s_o, s_e);
-        else tile_body(I1{}, I2{}, std::false_type{}, it, s_e, s_o);
+        if (it & 1) tile_body(I3{}, I0{}, std::false_type{}, it, s_o, s_e, 0, 0);
+        else tile_body(I1{}, I2{}, std::false_type{}, it, s_e, s_o, 0, 0);
       }
       if (it & 1) softmax_only(s_o); else softmax_only(s_e);
       wait_vmcnt<0>();
@@ -569,10 +599,10 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
       // tile it+1 sits in K slot (it+1)&3
       for (; it + 1 < ntiles; ++it) {
         switch ((it + 1) & 3) {
-          case 0: tile_body(I0{}, I0{}, std::false_type{}, it, s_e, s_o); break;
-          case 1: tile_body(I1{}, I0{}, std::false_type{}, it, s_e, s_o); break;
-          case 2: tile_body(I2{}, I0{}, std::false_type{}, it, s_e, s_o); break;
-          default: tile_body(I3{}, I0{}, std::false_type{}, it, s_e, s_o); break;
+          case 0: tile_body(I0{}, I0{}, std::false_type{}, it, s_e, s_o, 0, 0); break;
+          case 1: tile_body(I1{}, I0{}, std::false_type{}, it, s_e, s_o, 0, 0); break;
+          case 2: tile_body(I2{}, I0{}, std::false_type{}, it, s_e, s_o, 0, 0); break;
+          default: tile_body(I3{}, I0{}, std::false_type{}, it, s_e, s_o, 0, 0); break;
         }
 #pragma unroll
         for (int mb = 0; mb < NMB; ++mb) s_e[mb] = s_o[mb];
@@ -616,19 +646,37 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   }
 
   // ---- epilogue --------------------------------------------------------------------
+  // The wave's 32 x D output tile is one contiguous piece of O.  It is turned from "a lane
+  // holds a row" into "a lane holds 16 consecutive bytes" through a wave-private piece of
+  // LDS (row pitch + 8 bytes: conflict-free both ways), so that every store instruction
+  // writes whole cache lines.
   if constexpr (HAS_V) {
-    if (qrow_ok) {
-      const float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
-      uint16_t* orow = p.o + head_off + (size_t)qrow * D;
+    constexpr int RS = ROWB + 8;
+    constexpr int EP0 = (KSPLIT == 2) ? Cfg::kMerge : 0;
+    static_assert(EP0 + NQW * 32 * RS <= Cfg::kRing, "output staging must fit the ring");
+    unsigned char* ep = smem + EP0 + qsub * 32 * RS;
+    const float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
 #pragma unroll
-      for (int db = 0; db < NDB; ++db)
+    for (int db = 0; db < NDB; ++db)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          u32x2 w;
-          w[0] = pack_bf16(oacc[db][4 * j + 0] * inv, oacc[db][4 * j + 1] * inv);
-          w[1] = pack_bf16(oacc[db][4 * j + 2] * inv, oacc[db][4 * j + 3] * inv);
-          *reinterpret_cast<u32x2*>(orow + 32 * db + 8 * j + 4 * g) = w;
-        }
+      for (int j = 0; j < 4; ++j) {
+        u32x2 w;
+        w[0] = pack_bf16(oacc[db][4 * j + 0] * inv, oacc[db][4 * j + 1] * inv);
+        w[1] = pack_bf16(oacc[db][4 * j + 2] * inv, oacc[db][4 * j + 3] * inv);
+        *reinterpret_cast<u32x2*>(ep + ln * RS + (32 * db + 8 * j + 4 * g) * 2) = w;
+      }
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    constexpr int RPI = 64 / CPR;     // rows per store instruction
+    const int er = lane / CPR, ec = lane % CPR;
+    uint16_t* otile = p.o + head_off + (size_t)q0 * D;
+#pragma unroll
+    for (int i = 0; i < 32 / RPI; ++i) {
+      const int row = i * RPI + er;
+      const u32x2 lo = *reinterpret_cast<const u32x2*>(ep + row * RS + ec * 16);
+      const u32x2 hi = *reinterpret_cast<const u32x2*>(ep + row * RS + ec * 16 + 8);
+      const u32x4 w = {lo[0], lo[1], hi[0], hi[1]};
+      if (q0 + row < p.S) *reinterpret_cast<u32x4*>(otile + (size_t)row * D + ec * 8) = w;
     }
   }
   if (g == 0) {
