@@ -27,15 +27,17 @@
 // V^T operand comes from ds_read_b64_tr_b16, which hands lane j of a 16-lane group the
 // j-th 16-bit column of the 4 rows the group addressed.
 //
-// Schedule.  Tiles are consumed in "phases" K0 | K1 V0 | K2 V1 | ... : the scores of tile
-// i+1 are multiplied while the softmax of tile i runs on the vector ALU, and the row
-// maxima of tile i+1 are reduced while P_i V_i is multiplied.  Phase j lives in ring slot
-// j & 3; every phase is  wait (own loads of this phase) -> barrier -> issue phase j+3 into
-// the slot the barrier just freed -> multiply.  The steady-state loop is unrolled over two
-// tiles so that every slot is a compile-time constant: LDS addresses are a per-lane base
-// plus an instruction immediate, the wait counts are literals, and the loop carries almost
-// no scalar or address arithmetic - the instruction issue rate, not the matrix pipe, is
-// what bounds this kernel.
+// Schedule.  One barrier per tile.  Between the barriers of tile i a wave multiplies the
+// scores of tile i+1 while the softmax of tile i runs on the vector ALU, then P_i V_i while
+// the row maxima of tile i+1 are reduced; the V^T operands are requested from LDS while
+// the last score multiplies run, so the 16 (or 32) multiplies of a tile form one
+// uninterrupted run.  The ring has three K slots and two V slots (5 x 16 KB at d = 128: two
+// workgroups fill the 160 KB of a CU): the barrier of tile i frees the slots of K(i) and
+// V(i-1), and V(i+1) and K(i+3) are copied into them, their issue spread between the
+// multiplies.  The steady-state loop is unrolled over six tiles so that every slot is a
+// compile-time constant: LDS addresses are a per-lane base plus an instruction immediate,
+// the wait counts are literals, and the loop carries almost no scalar or address
+// arithmetic - instruction issue and latency, not the matrix pipe, bound this kernel.
 #pragma once
 #include <type_traits>
 
@@ -50,7 +52,11 @@ typedef SPATTN_LDS const unsigned char* lds_cptr;
 template <int D, int MODE, bool HAS_V>
 struct AttnCfg {
   static constexpr int kTileBytes = 64 * D * 2;
-  static constexpr int kSlots = 4;
+  // Ring slots: K tiles are copied three tiles ahead (two with token lists, whose key
+  // validity ring shares the 80 KB that let two workgroups share a CU), V tiles one ahead.
+  static constexpr int kKSlots = (MODE == KV_TOKENS) ? 2 : 3;
+  static constexpr int kVSlots = HAS_V ? 2 : 0;
+  static constexpr int kSlots = kKSlots + kVSlots;
   static constexpr int kBiasRing = 8;                         // tiles of key-validity bias (token lists)
   static constexpr int kBiasBytes = (MODE == KV_TOKENS) ? kBiasRing * 64 * 4 : 0;
   static constexpr int kRing = kSlots * kTileBytes;
@@ -68,8 +74,14 @@ __device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(gptr) : "memory");
 }
 // Same with a wave-uniform base pointer and a 32-bit per-lane byte offset.
+// The base goes through readfirstlane: under scalar-register pressure the compiler may keep
+// a uniform pointer in vector registers, which the "s" constraint alone does not undo.
 __device__ __forceinline__ void dma16(const void* sbase, uint32_t voff, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(voff), "s"(sbase) : "memory");
+  const uint64_t b = (uint64_t)(uintptr_t)sbase;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)b);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
+  const uint64_t sb = ((uint64_t)hi << 32) | lo;
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(voff), "s"(sb) : "memory");
 }
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
@@ -92,6 +104,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   constexpr int TILE = Cfg::kTileBytes;
   constexpr int LPT = Cfg::kLoadsPerTile;
   constexpr int RPL = Cfg::kRowsPerLoad;
+  constexpr int NK = Cfg::kKSlots;
   constexpr float kNegInf = -__builtin_huge_valf();
 
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
@@ -133,9 +146,6 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     ntiles = (MODE == KV_TOKENS) ? ((n + 63) >> 6) : n;
   }
   const int last_row = p.kv_len - 1;
-  // Phase numbers: with V, 0 = K0, 2i+1 = K(i+1), 2i+2 = V(i); phase 2*ntiles-1 would be a
-  // K tile past the end and is never issued.  Without V, phase j = K(j).
-  const int last_phase = HAS_V ? 2 * ntiles : ntiles - 1;
 
   // ---- loader role: load i of a tile covers rows RPL*(4i + wave) .. +RPL-1 ----------
   const int ld_sub = lane / CPR;       // row within the load
@@ -149,27 +159,40 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   auto swz = [](int r) -> int {
     return D == 128 ? (((r & 3) << 2) | ((r >> 2) & 3)) : ((((r >> 1) & 1) << 2) | ((r >> 2) & 3));
   };
-  auto ld_row = [&](int i) -> int { return RPL * (4 * i + wave) + ld_sub; };
-  auto ld_off = [&](int i) -> int { return (ld_slot ^ swz(ld_row(i))) << 4; };   // chunk offset within the row
+  // The loads of a tile are 4 RPL rows apart, a multiple of the swizzle period: one chunk
+  // offset serves all of them.
+  static_assert((4 * RPL) % 16 == 0, "loads of one wave must share the swizzle");
+  const int ld_row0 = RPL * wave + ld_sub;
+  const int ld_off0 = (ld_slot ^ swz(ld_row0)) << 4;   // chunk offset within the row
+  auto ld_row = [&](int i) -> int { return ld_row0 + 4 * RPL * i; };
+  auto ld_off = [&](int) -> int { return ld_off0; };
   uint32_t ld_go[LPT];                 // lane offset within a contiguous 64-row tile
 #pragma unroll
-  for (int i = 0; i < LPT; ++i) ld_go[i] = ld_row(i) * ROWB + ld_off(i);
+  for (int i = 0; i < LPT; ++i) {
+    // a key sequence shorter than one tile: rows past its end re-read the last row
+    const int row = ld_row(i) > last_row ? last_row : ld_row(i);
+    ld_go[i] = row * ROWB + ld_off0;
+  }
 
-  // First key row of a tile (dense / block lists) from its id; kv_len marks "no such block".
-  // The id of tile t is t itself (dense) or the t-th list entry (block lists).
-  auto tile_id = [&](int t) -> int {
-    if constexpr (MODE == KV_BLOCKS) return lst[t];
-    return t;
-  };
-  auto id_row0 = [&](int blk) -> int {
-    if constexpr (MODE == KV_DENSE) return blk * 64;
-    if constexpr (MODE == KV_BLOCKS) return (blk >= 0 && blk <= (last_row >> 6)) ? blk * 64 : p.kv_len;
-    return 0;
-  };
-  // Same, for a tile that may lie past the end of the list (prefetched ids that are never used).
-  auto tile_id_clamped = [&](int t) -> int {
-    if constexpr (MODE == KV_BLOCKS) return lst[t < p.idx_stride ? t : p.idx_stride - 1];
-    return t;
+  // Dense / block lists: a tile is described by the first row that is copied and by how
+  // many of its 64 keys exist, packed as  start | keys << 24  (wave-uniform, one SGPR).
+  // A tile that runs past kv_len is copied as the LAST 64 rows of the sequence, so that no
+  // lane needs a row clamp of its own: its keys then sit at the end of the tile and the
+  // rows in front of them (keys of the previous block) are masked.  A sequence shorter than
+  // one tile is copied from row 0 with the clamped lane offsets above.  A block id outside
+  // the sequence describes a tile with no keys.
+  // The id of tile t is t itself (dense) or the t-th list entry (block lists); positions
+  // past the end of the list may be asked for (prefetch), their descriptors are never used.
+  const bool kv_short = p.kv_len < 64;
+  auto tile_desc = [&](int t) -> int {
+    int id = t;
+    if constexpr (MODE == KV_BLOCKS) id = lst[t < p.idx_stride ? t : p.idx_stride - 1];
+    const bool valid = id >= 0 && id <= (last_row >> 6);
+    const int r0 = valid ? id * 64 : 0;
+    int keys = valid ? p.kv_len - r0 : 0;
+    keys = keys > 64 ? 64 : keys;
+    const int start = (keys < 64 && !kv_short) ? p.kv_len - 64 : r0;
+    return start | (keys << 24);
   };
 
   // Token lists: the RPL token ids behind one load are wave-uniform, so they are fetched
@@ -208,13 +231,13 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
 
   // Loads of one K or V tile into ring slot `slot`: prepare() resolves the wave-uniform
   // base and this lane's byte offsets, load(i) issues the i-th of the LPT wave-wide copies.
-  // Issue order of the tiles is K0 K1 V0 K2 V1 ..., which the token-row queue relies on.
+  // With token lists the tiles are issued K0 K1 V0 K2 V1 ..., which the token-row queue relies on.
   struct TileLoad {
     const unsigned char* base;
     uint32_t lds;
     uint32_t go[LPT];
   };
-  auto prepare_tile = [&](int t, int id, int slot, bool is_v) -> TileLoad {
+  auto prepare_tile = [&](int t, int desc, int slot, bool is_v) -> TileLoad {
     TileLoad tl;
     tl.lds = smem_base + (uint32_t)slot * TILE + wave * 1024;
     const unsigned char* src = is_v ? vh : kh;
@@ -240,52 +263,17 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
         tok_fetch(t + 2);
       }
     } else {
-      const int r0 = id_row0(id);
-      if (r0 + 64 <= p.kv_len) {
-        tl.base = src + (size_t)r0 * ROWB;   // whole tile in range
+      tl.base = src + (size_t)(desc & 0xffffff) * ROWB;
 #pragma unroll
-        for (int i = 0; i < LPT; ++i) tl.go[i] = ld_go[i];
-      } else {
-        // ragged last tile: rows past the end re-read the last row and are masked later
-        tl.base = src;
-#pragma unroll
-        for (int i = 0; i < LPT; ++i) {
-          int row = r0 + ld_row(i);
-          row = row > last_row ? last_row : row;
-          tl.go[i] = (uint32_t)row * ROWB + ld_off(i);
-        }
-      }
+      for (int i = 0; i < LPT; ++i) tl.go[i] = ld_go[i];
     }
     return tl;
   };
   auto load_part = [&](const TileLoad& tl, int i) { dma16(tl.base, tl.go[i], tl.lds + i * 4096); };
   auto issue_tile = [&](int t, int slot, bool is_v) {
-    const TileLoad tl = prepare_tile(t, tile_id(t), slot, is_v);
+    const TileLoad tl = prepare_tile(t, tile_desc(t), slot, is_v);
 #pragma unroll
     for (int i = 0; i < LPT; ++i) load_part(tl, i);
-  };
-  auto phase_exists = [&](int j) -> bool {
-    if (j > last_phase) return false;
-    if constexpr (HAS_V) return j != 2 * ntiles - 1;
-    return true;
-  };
-  // Generic form: issue phase j if it exists.
-  auto issue_phase = [&](int j) {
-    if (!phase_exists(j)) return;
-    if constexpr (HAS_V) {
-      if (j == 0) issue_tile(0, 0, false);
-      else if (j & 1) issue_tile((j + 1) / 2, j & 3, false);
-      else issue_tile(j / 2 - 1, j & 3, true);
-    } else {
-      issue_tile(j, j & 3, false);
-    }
-  };
-  // Generic wait for phase j: phases j+1 and j+2, if they exist, may stay in flight.
-  auto wait_generic = [&](int j) {
-    const int later = (phase_exists(j + 1) ? 1 : 0) + (phase_exists(j + 2) ? 1 : 0);
-    if (later == 2) wait_vmcnt<2 * LPT>();
-    else if (later == 1) wait_vmcnt<LPT>();
-    else wait_vmcnt<0>();
   };
 
   // ---- prologue ------------------------------------------------------------------
@@ -293,10 +281,15 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   const int qrow = q0 + ln;
   const bool qrow_ok = qrow < p.S;
 
+  auto kslot = [](int t) -> int { return t % NK; };
+  auto vslot = [](int t) -> int { return NK + (t & 1); };
+
+  // Copies go out in the order K0 K1 V0 K2 | V1 K3 | V2 K4 | ... (three K slots) or
+  // K0 K1 V0 | K2 V1 | K3 V2 | ... (two K slots, token lists).
   tok_fetch(0);
   tok_resolve(0);
   tok_fetch(1);
-  issue_phase(0);
+  if (ntiles > 0) issue_tile(0, kslot(0), false);
   // The Q loads are the only compiler-visible vector loads of the kernel.  They go out
   // between the first copies so that their latency overlaps that of tile 0, and must have
   // retired before the first counted wait.
@@ -306,8 +299,12 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     const u32x4 z = {0, 0, 0, 0};
     qf[t] = qrow_ok ? *reinterpret_cast<const u32x4*>(qh + (size_t)qrow * D + 16 * t + 8 * g) : z;
   }
-  issue_phase(1);
-  issue_phase(2);
+  int head_pending = 0;   // tile copies behind K0 when the first phase waits
+  if (ntiles > 0) {
+    if (1 < ntiles) { issue_tile(1, kslot(1), false); ++head_pending; }
+    if constexpr (HAS_V) { issue_tile(0, vslot(0), true); ++head_pending; }
+    if (NK == 3 && 2 < ntiles) { issue_tile(2, kslot(2), false); ++head_pending; }
+  }
 #pragma unroll
   for (int t = 0; t < NT; ++t) asm volatile("" ::"v"(qf[t]));
 
@@ -340,24 +337,30 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   // Transposing V read: in each 16-lane group, lane i addresses 4 dims of key (i>>2);
   // lane j receives dim j of those 4 keys.  Keys 4g..4g+3 (+8 for the second read) of
   // each 16-key step, dims 32db + 16*dhalf + 4*(i&3)..+3.
-  lds_cptr v_lo[HAS_V ? NDB : 1];    // keys 4g..4g+3 of a step
-  lds_cptr v_lo2[HAS_V ? NDB : 1];   // keys 8+4g..8+4g+3 of a step (their rows have another swizzle)
+  // All V addresses of a lane derive from one: the 32-dim block db sits in chunk bits 2-3,
+  // which the swizzle only XORs (address ^ (db << 6)), and rows r and r+8 differ in one
+  // swizzle bit (address ^ 32, + 8 rows).  They are re-derived per tile instead of being
+  // kept in eight registers.
+  uint32_t v_base = 0, v_cur = 0;
   if constexpr (HAS_V) {
     const int i16 = lane & 15;
     const int dhalf = (lane >> 4) & 1;
     const int r1 = ksub * KW + 4 * g + (i16 >> 2);
     const int cb = 2 * dhalf + ((i16 & 3) >> 1);
-#pragma unroll
-    for (int db = 0; db < NDB; ++db) {
-      v_lo[db] = smem_l + r1 * ROWB + (((4 * db + cb) ^ swz(r1)) << 4) + ((i16 & 1) << 3);
-      v_lo2[db] = smem_l + (r1 + 8) * ROWB + (((4 * db + cb) ^ swz(r1 + 8)) << 4) + ((i16 & 1) << 3);
-    }
+    static_assert(NDB <= 4, "db must fit chunk bits 2-3");
+    // relative to the first V slot: instruction offsets reach 64 KB, the ring is larger
+    v_base = smem_base + NK * TILE + r1 * ROWB + ((cb ^ swz(r1)) << 4) + ((i16 & 1) << 3);
   }
+  // Called once per tile: hides v_base from loop-invariant code motion.
+  auto v_addr_refresh = [&]() {
+    v_cur = v_base;
+    asm volatile("" : "+v"(v_cur));
+  };
 
   // ---- building blocks --------------------------------------------------------------
   // Keys of tile `it` that do not exist get -inf.  Accumulator register 4j+i of block mb
   // is key ksub*KW + 32mb + 8j + 4g + i of the tile.
-  auto mask_tile = [&](int it, int id, f32x16 (&s)[NMB]) {
+  auto mask_tile = [&](int it, int desc, f32x16 (&s)[NMB]) {
     if constexpr (MODE == KV_TOKENS) {
       const float* bias = reinterpret_cast<const float*>(smem + Cfg::kTotal - Cfg::kBiasBytes) + (it % Cfg::kBiasRing) * 64;
 #pragma unroll
@@ -371,28 +374,41 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
           s[mb][4 * j + 3] += bv.w;
         }
     } else {
-      const int r0 = id_row0(id);
-      if (r0 + 64 > p.kv_len) {
+      const int keys = desc >> 24;
+      if (keys < 64) {
+        // existing keys are tile rows lo .. hi-1 (wave-uniform)
+        const int lo = kv_short ? 0 : 64 - keys;
+        const int hi = kv_short ? keys : 64;
+        const int kb = ksub * KW + 4 * g;    // this lane's first key
 #pragma unroll
         for (int mb = 0; mb < NMB; ++mb)
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-            const int key = r0 + ksub * KW + 32 * mb + 8 * (r >> 2) + 4 * g + (r & 3);
-            if (key >= p.kv_len) s[mb][r] = kNegInf;
+            const int c = 32 * mb + 8 * (r >> 2) + (r & 3);
+            if (kb < lo - c || kb >= hi - c) s[mb][r] = kNegInf;
           }
       }
     }
   };
-  // Row max of a score tile (both 32-lane halves); returns max * sf.
-  auto row_stats = [&](const f32x16 (&s)[NMB]) -> float {
-    float mloc = s[0][0];
-#pragma unroll
-    for (int mb = 0; mb < NMB; ++mb)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) mloc = fmaxf(mloc, s[mb][r]);
+  // Row max of a score tile in NP pieces (so that they can be placed between multiplies),
+  // then the exchange between the two 32-lane halves; returns max * sf.
+  constexpr int NP = 4 * NMB;
+  auto stat_piece = [&](const f32x16 (&s)[NMB], int k, float& mloc) {
+    const int mb = k >> 2, r = 4 * (k & 3);
+    if (k == 0) mloc = s[0][0];
+    mloc = fmaxf(mloc, fmaxf(s[mb][r], s[mb][r + 1]));
+    mloc = fmaxf(mloc, fmaxf(s[mb][r + 2], s[mb][r + 3]));
+  };
+  auto stat_finish = [&](float mloc) -> float {
     mloc = pair_max(mloc);
     m_true = fmaxf(m_true, mloc);
     return mloc * p.sf;
+  };
+  auto row_stats = [&](const f32x16 (&s)[NMB]) -> float {
+    float mloc;
+#pragma unroll
+    for (int k = 0; k < NP; ++k) stat_piece(s, k, mloc);
+    return stat_finish(mloc);
   };
   // Move the exponent reference if some row of the wave outgrew it; rescales O and l.
   auto maybe_rescale = [&](float mloc_sf) {
@@ -423,8 +439,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     }
   };
   // Pin the softmax results where they are produced; otherwise the compiler sinks the
-  // whole softmax to the first use of P, behind the next barrier, and nothing overlaps
-  // the MFMAs.
+  // whole softmax to the first use of P and nothing overlaps the MFMAs.
   auto pin_softmax = [&]() {
     asm volatile("" : "+v"(l_run));
     if constexpr (HAS_V) {
@@ -439,175 +454,210 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
 #pragma unroll
     for (int mb = 0; mb < NMB; ++mb) softmax_chunk(s, base, mb, 0, 16);
   };
+
+  // V^T operands of one 16-key step (PV group gi = 2mb + h), double-buffered over groups.
+  constexpr int NG = 2 * NMB;
+  u32x2 va[HAS_V ? 2 : 1][HAS_V ? NDB : 1][2];
+  auto v_reads = [&](uint32_t vofs, int gi) {
+    if constexpr (HAS_V) {
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) {
+        const uint32_t x1 = v_cur ^ (uint32_t)(db << 6);
+        const uint32_t x2 = x1 ^ 32u;
+        const lds_cptr a1 = (lds_cptr)(uintptr_t)x1 + vofs + gi * 16 * ROWB;
+        const lds_cptr a2 = (lds_cptr)(uintptr_t)x2 + vofs + gi * 16 * ROWB + 8 * ROWB;
+        va[gi & 1][db][0] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((SPATTN_LDS s16x4*)a1));
+        va[gi & 1][db][1] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((SPATTN_LDS s16x4*)a2));
+      }
+    }
+  };
+
   // s_out^T = K Q^T from the K tile at ring offset kofs (bytes), one 32-key block at a
-  // time; if WITH_SM, the softmax of s_in is interleaved: one MFMA, then the vector-ALU
-  // work of 16/NT score registers.
-  auto qk_tile = [&](auto with_sm, uint32_t kofs, f32x16 (&s_out)[NMB], f32x16 (&s_in)[NMB], const TileLoad* tl) {
+  // time.  WITH_SM: the softmax of s_in is interleaved, one MFMA then the vector-ALU work of
+  // 16/NT score registers.  tl: a tile copy whose parts are issued between the multiplies
+  // if `live` (in one burst they queue behind the other waves' copies and stall this wave).
+  // EARLY_V: the V^T operands of the first PV group are requested before the last multiply,
+  // so that PV does not start by waiting for LDS.
+  constexpr int kEarly = 1;
+  auto qk_tile = [&](auto with_sm, auto early_v, uint32_t kofs, uint32_t vofs, f32x16 (&s_out)[NMB], f32x16 (&s_in)[NMB],
+                     const TileLoad* tl, bool live) {
     constexpr bool WITH_SM = decltype(with_sm)::value;
+    constexpr bool EARLY_V = decltype(early_v)::value;
     constexpr int EPM = 16 / NT;
     const float base = (mr_sf == kNegInf) ? 0.f : mr_sf;
 #pragma unroll
     for (int mb = 0; mb < NMB; ++mb) {
       u32x4 ka[NT];
+      auto k_reads = [&](int t0, int t1) {
 #pragma unroll
-      for (int t = 0; t < NT; ++t) ka[t] = *(SPATTN_LDS const u32x4*)(k_lo[t] + kofs + mb * 32 * ROWB);
-      __builtin_amdgcn_sched_barrier(0);   // all reads in flight before the first multiply
+        for (int t = t0; t < t1; ++t) ka[t] = *(SPATTN_LDS const u32x4*)(k_lo[t] + kofs + mb * 32 * ROWB);
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      // the operands arrive in two batches, to bound the registers they hold
+      k_reads(0, NT / 2);
+      const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      auto steps = [&](int t0, int t1) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) s_out[mb][r] = 0.f;
-#pragma unroll
-      for (int t = 0; t < NT; ++t) {
-        s_out[mb] = mfma32(ka[t], qf[t], s_out[mb]);
-        if constexpr (WITH_SM) softmax_chunk(s_in, base, mb, t * EPM, EPM);
-        // the next tile's copies are spread over the multiplies: issued in one burst they
-        // queue behind the other waves' copies and stall this wave
-        if (tl != nullptr) {
-          constexpr int STEP = (NMB * NT) / LPT;
-          const int m = mb * NT + t;
-          if (m % STEP == STEP - 1) load_part(*tl, m / STEP);
+        for (int t = t0; t < t1; ++t) {
+          s_out[mb] = mfma32(ka[t], qf[t], t == 0 ? zero : s_out[mb]);
+          if constexpr (WITH_SM) softmax_chunk(s_in, base, mb, t * EPM, EPM);
+          if (tl != nullptr && live) {
+            constexpr int STEP = (NMB * NT) / LPT;
+            const int m = mb * NT + t;
+            if (m % STEP == STEP - 1) load_part(*tl, m / STEP);
+          }
         }
-      }
-      if constexpr (WITH_SM) {
+        if constexpr (WITH_SM) {
 #pragma unroll
-        for (int t = 0; t < NT; ++t) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);            // one MFMA
-          __builtin_amdgcn_sched_group_barrier(0x002, EPM * 7 / 2, 0);  // its share of the softmax
+          for (int t = t0; t < t1; ++t) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);            // one MFMA
+            __builtin_amdgcn_sched_group_barrier(0x002, EPM * 7 / 2, 0);  // its share of the softmax
+          }
         }
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      steps(0, NT / 4);
+      k_reads(NT / 2, NT);
+      if (EARLY_V && mb == NMB - 1) {
+        steps(NT / 4, NT - kEarly);
+        v_reads(vofs, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        steps(NT - kEarly, NT);
+      } else {
+        steps(NT / 4, NT);
       }
-      __builtin_amdgcn_sched_barrier(0);
     }
     if constexpr (WITH_SM) pin_softmax();
   };
-  // O^T += V^T P^T from the V tile at ring offset vofs, two 16-key steps at a time.
-  auto pv_tile = [&](uint32_t vofs, const TileLoad* tl) {
+  // O^T += V^T P^T from the V tile at offset vofs from the first V slot, one 16-key step (NDB multiplies) at
+  // a time; the operands of step 0 are in flight or here already (FIRST_LOADED), those of
+  // step gi+1 are requested before step gi is multiplied.  STAT: the row maxima of s_next
+  // are reduced between the multiplies; returns them (times sf).
+  auto pv_tile = [&](auto first_loaded, auto stat_c, uint32_t vofs, const TileLoad* tl, bool live, const f32x16 (&s_next)[NMB]) -> float {
+    constexpr bool STAT = decltype(stat_c)::value;
+    float mloc = 0.f;
     if constexpr (HAS_V) {
+      if constexpr (!decltype(first_loaded)::value) v_reads(vofs, 0);
 #pragma unroll
-      for (int mb = 0; mb < NMB; ++mb) {
-        u32x2 va[2][NDB][2];
-#pragma unroll
-        for (int h = 0; h < 2; ++h)
-#pragma unroll
-          for (int db = 0; db < NDB; ++db) {
-            const lds_cptr a1 = v_lo[db] + vofs + (2 * mb + h) * 16 * ROWB;
-            const lds_cptr a2 = v_lo2[db] + vofs + (2 * mb + h) * 16 * ROWB;
-            va[h][db][0] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((SPATTN_LDS s16x4*)a1));
-            va[h][db][1] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((SPATTN_LDS s16x4*)a2));
-          }
+      for (int gi = 0; gi < NG; ++gi) {
+        if (gi + 1 < NG) v_reads(vofs, gi + 1);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
+        for (int db = 0; db < NDB; ++db) {
+          const u32x4 a = {va[gi & 1][db][0][0], va[gi & 1][db][0][1], va[gi & 1][db][1][0], va[gi & 1][db][1][1]};
+          oacc[db] = mfma32(a, pb[gi], oacc[db]);
+          const int m = gi * NDB + db;
+          if constexpr (STAT) {
+            constexpr int PPM = (NP + NG * NDB - 1) / (NG * NDB);   // pieces per multiply
 #pragma unroll
-          for (int db = 0; db < NDB; ++db) {
-            const u32x4 a = {va[h][db][0][0], va[h][db][0][1], va[h][db][1][0], va[h][db][1][1]};
-            oacc[db] = mfma32(a, pb[2 * mb + h], oacc[db]);
-            if (tl != nullptr) {   // the next tile's copies, spread over the multiplies
-              constexpr int STEP = (NMB * 2 * NDB) / LPT;
-              const int m = (mb * 2 + h) * NDB + db;
-              if (m % STEP == STEP - 1) load_part(*tl, m / STEP);
-            }
+            for (int k = m * PPM; k < (m + 1) * PPM && k < NP; ++k) stat_piece(s_next, k, mloc);
           }
+          if (tl != nullptr && live) {   // a tile copy, spread over the multiplies
+            constexpr int STEP = (NG * NDB) / LPT;
+            if (m % STEP == STEP - 1) load_part(*tl, m / STEP);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
       }
+    } else if constexpr (STAT) {
+#pragma unroll
+      for (int k = 0; k < NP; ++k) stat_piece(s_next, k, mloc);
     }
+    if constexpr (STAT) return stat_finish(mloc);
+    return 0.f;
   };
 
-  // One tile of the pipeline: K phase of tile it+1 (ring slot KS) with the softmax of tile
-  // it (scores in s_a), then V phase of tile it (ring slot VS) with the row maxima of tile
-  // it+1 (scores in s_b).  In the steady state every later phase exists, so waits and
-  // issues are unconditional.
-  // id_v / id_k: ids of tiles it+1 and it+3 (it+4 without V), fetched ahead of time by the
-  // steady loop so that no list load sits between a barrier and the copies behind it;
-  // the generic form looks them up itself.
-  auto tile_body = [&](auto ks_c, auto vs_c, auto steady_c, int it, f32x16 (&s_a)[NMB], f32x16 (&s_b)[NMB], int id_v, int id_k) {
-    constexpr int KS = decltype(ks_c)::value;
-    constexpr int VS = decltype(vs_c)::value;
-    constexpr bool STEADY = decltype(steady_c)::value;
-    {
-      const int j = HAS_V ? 2 * it + 1 : it + 1;
-      if constexpr (STEADY) wait_vmcnt<2 * LPT>(); else wait_generic(j);
-      __syncthreads();
-      // phase j+3 is V(it+1) (with V) or K(it+4)
-      if constexpr (STEADY) {
-        const TileLoad tl = HAS_V ? prepare_tile(it + 1, id_v, (VS + 2) & 3, true) : prepare_tile(it + 4, id_k, (KS + 3) & 3, false);
-        qk_tile(std::true_type{}, KS * TILE, s_b, s_a, &tl);
-      } else {
-        if constexpr (HAS_V) {
-          if (it + 1 < ntiles) issue_tile(it + 1, (VS + 2) & 3, true);
-        } else {
-          if (it + 4 < ntiles) issue_tile(it + 4, (KS + 3) & 3, false);
-        }
-        qk_tile(std::true_type{}, KS * TILE, s_b, s_a, nullptr);
-      }
-      mask_tile(it + 1, STEADY ? id_v : tile_id(it + 1), s_b);
-    }
+  f32x16 s_e[NMB], s_o[NMB];   // scores of even / odd tiles
+  int idw[6] = {0, 0, 0, 0, 0, 0};   // descriptors of tiles it+1 .. it+NK(+1), tile j in idw[j % 6]
+
+  // One tile of the pipeline, between two barriers: the scores of tile it+1 are multiplied
+  // (K slot (it+1) % NK) while the softmax of tile it runs on the vector ALU, then P V of
+  // tile it (V slot NK + it % 2) is multiplied while the row maxima of tile it+1 are
+  // reduced.  The barrier frees the slots of K(it) and V(it-1): V(it+1) and, if it exists,
+  // K(it+NK) are copied into them.  KC = it % 6 fixes every slot at compile time.
+  auto tile_body = [&](auto kc, int it) {
+    constexpr int KC = decltype(kc)::value;
+    // KS, KN: ring slots of K(it+1), K(it+NK); VS: V slot of tile it counted from the first
+    // V slot; VN: ring slot of V(it+1)
+    constexpr int KS = (KC + 1) % NK, VS = KC % 2, KN = KC % NK, VN = NK + (KC + 1) % 2;
+    auto& s_a = (KC & 1) ? s_o : s_e;   // tile it
+    auto& s_b = (KC & 1) ? s_e : s_o;   // tile it+1
+    const bool has_kn = it + NK < ntiles;
+    // behind K(it+1) and V(it) only K(it+2) can be in flight (three K slots)
+    if (NK == 3 && it + 2 < ntiles) wait_vmcnt<LPT>(); else wait_vmcnt<0>();
+    __syncthreads();
+    v_addr_refresh();
+    const int d_v = idw[(KC + 1) % 6];
+    const int d_k = idw[(KC + NK) % 6];
+    constexpr bool K_FIRST = (MODE == KV_TOKENS) || !HAS_V;   // token rows are queued K first
+    const TileLoad tl_first = K_FIRST ? prepare_tile(it + NK, d_k, KN, false) : prepare_tile(it + 1, d_v, VN, true);
+    qk_tile(std::true_type{}, std::integral_constant<bool, HAS_V>{}, KS * TILE, VS * TILE, s_b, s_a, &tl_first,
+            K_FIRST ? has_kn : true);
+    mask_tile(it + 1, d_v, s_b);
+    if constexpr (MODE != KV_TOKENS) idw[(KC + NK + 1) % 6] = tile_desc(it + NK + 1);
+    float mloc_sf;
     if constexpr (HAS_V) {
-      const int j = 2 * it + 2;
-      if constexpr (STEADY) wait_vmcnt<2 * LPT>(); else wait_generic(j);
-      __syncthreads();
-      // phase j+3 is K(it+3)
-      if constexpr (STEADY) {
-        const TileLoad tl = prepare_tile(it + 3, id_k, KS, false);
-        pv_tile(VS * TILE, &tl);
-      } else {
-        if (it + 3 < ntiles) issue_tile(it + 3, KS, false);
-        pv_tile(VS * TILE, nullptr);
-      }
+      const TileLoad tl_second = K_FIRST ? prepare_tile(it + 1, d_v, VN, true) : prepare_tile(it + NK, d_k, KN, false);
+      mloc_sf = pv_tile(std::true_type{}, std::true_type{}, VS * TILE, &tl_second, K_FIRST ? true : has_kn, s_b);
+    } else {
+      mloc_sf = pv_tile(std::true_type{}, std::true_type{}, 0, nullptr, false, s_b);
     }
-    maybe_rescale(row_stats(s_b));
+    maybe_rescale(mloc_sf);
   };
   using I0 = std::integral_constant<int, 0>;
   using I1 = std::integral_constant<int, 1>;
   using I2 = std::integral_constant<int, 2>;
   using I3 = std::integral_constant<int, 3>;
+  using I4 = std::integral_constant<int, 4>;
+  using I5 = std::integral_constant<int, 5>;
 
   if (ntiles > 0) {
-    f32x16 s_e[NMB], s_o[NMB];   // scores of even / odd tiles
-    // phase 0: scores of tile 0
-    wait_generic(0);
+    // head: scores of tile 0
+    if (head_pending == 3) wait_vmcnt<3 * LPT>();
+    else if (head_pending == 2) wait_vmcnt<2 * LPT>();
+    else if (head_pending == 1) wait_vmcnt<LPT>();
+    else wait_vmcnt<0>();
     __syncthreads();
-    issue_phase(3);
-    qk_tile(std::false_type{}, 0, s_e, s_e, nullptr);
-    mask_tile(0, tile_id(0), s_e);
+    qk_tile(std::false_type{}, std::false_type{}, 0, 0, s_e, s_e, nullptr, false);
+    mask_tile(0, tile_desc(0), s_e);
     maybe_rescale(row_stats(s_e));
 
     int it = 0;
+    if constexpr (MODE != KV_TOKENS) {
+#pragma unroll
+      for (int j = 1; j <= NK; ++j) idw[j] = tile_desc(j);
+    }
+    // Rounds of six tiles without side exits (the register allocator handles one plain
+    // back-edge far better than six exits), then up to five single tiles.
+    while (it + 6 < ntiles) {
+      tile_body(I0{}, it);
+      tile_body(I1{}, it + 1);
+      tile_body(I2{}, it + 2);
+      tile_body(I3{}, it + 3);
+      tile_body(I4{}, it + 4);
+      tile_body(I5{}, it + 5);
+      it += 6;
+    }
+    if (it + 1 < ntiles) {
+      tile_body(I0{}, it++);
+      if (it + 1 < ntiles) {
+        tile_body(I1{}, it++);
+        if (it + 1 < ntiles) {
+          tile_body(I2{}, it++);
+          if (it + 1 < ntiles) {
+            tile_body(I3{}, it++);
+            if (it + 1 < ntiles) tile_body(I4{}, it++);
+          }
+        }
+      }
+    }
+    // tail: softmax and P V of the last tile
+    if (it & 1) softmax_only(s_o); else softmax_only(s_e);
     if constexpr (HAS_V) {
-      // tile `it` has its next K tile in slot (2it+1)&3 and its V tile in slot (2it+2)&3
-      // w1..w3: ids of tiles it+1..it+3; two more are fetched per round, a round ahead
-      int w1 = 0, w2 = 0, w3 = 0;
-      if (4 < ntiles) {
-        w1 = tile_id(1);
-        w2 = tile_id(2);
-        w3 = tile_id(3);
-      }
-      for (; it + 4 < ntiles; it += 2) {
-        const int w4 = tile_id(it + 4);
-        const int w5 = tile_id_clamped(it + 5);
-        tile_body(I1{}, I2{}, std::true_type{}, it, s_e, s_o, w1, w3);
-        tile_body(I3{}, I0{}, std::true_type{}, it + 1, s_o, s_e, w2, w4);
-        w1 = w3;
-        w2 = w4;
-        w3 = w5;
-      }
-      for (; it + 1 < ntiles; ++it) {
-        if (it & 1) tile_body(I3{}, I0{}, std::false_type{}, it, s_o, s_e, 0, 0);
-        else tile_body(I1{}, I2{}, std::false_type{}, it, s_e, s_o, 0, 0);
-      }
-      if (it & 1) softmax_only(s_o); else softmax_only(s_e);
       wait_vmcnt<0>();
       __syncthreads();
-      pv_tile((uint32_t)((2 * ntiles) & 3) * TILE, nullptr);
-    } else {
-      // tile it+1 sits in K slot (it+1)&3
-      for (; it + 1 < ntiles; ++it) {
-        switch ((it + 1) & 3) {
-          case 0: tile_body(I0{}, I0{}, std::false_type{}, it, s_e, s_o, 0, 0); break;
-          case 1: tile_body(I1{}, I0{}, std::false_type{}, it, s_e, s_o, 0, 0); break;
-          case 2: tile_body(I2{}, I0{}, std::false_type{}, it, s_e, s_o, 0, 0); break;
-          default: tile_body(I3{}, I0{}, std::false_type{}, it, s_e, s_o, 0, 0); break;
-        }
-#pragma unroll
-        for (int mb = 0; mb < NMB; ++mb) s_e[mb] = s_o[mb];
-      }
-      softmax_only(s_e);
+      v_addr_refresh();
+      pv_tile(std::false_type{}, std::false_type{}, (uint32_t)(it & 1) * TILE, nullptr, false, s_e);
     }
   }
   __syncthreads();   // every wave is done with the ring
