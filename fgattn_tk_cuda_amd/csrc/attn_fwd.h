@@ -314,10 +314,18 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   // exceed 1 (by at most 2^kSlack), which fp32 sums and bf16 P hold without loss, and the
   // O / l rescale is skipped on most tiles.  m_true tracks the true raw max for the
   // statistics outputs.
+  // Without statistics outputs the row maxima are not even computed per tile (LAZY_MAX):
+  // a row that outgrew the reference shows in the tile's own sum of p (above 2^kSlack, inf
+  // or NaN), and only then are the maxima taken, the reference moved and the tile's
+  // exponentials redone.
   constexpr float kSlack = 8.f;
+  constexpr float kTrigger = 256.f;   // 2^kSlack
+  constexpr bool LAZY_MAX = !STATS;
   float mr_sf = kNegInf;
+  float base_eff = 0.f;    // mr_sf, or 0 while no key has been seen
   float m_true = kNegInf;
   float l_run = 0.f;       // running denominator, this lane's keys only
+  float l_tile = 0.f;      // sum of p over the tile whose softmax is in progress
   f32x16 oacc[HAS_V ? NDB : 1];
 #pragma unroll
   for (int db = 0; db < (HAS_V ? NDB : 1); ++db)
@@ -352,9 +360,10 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     v_base = smem_base + NK * TILE + r1 * ROWB + ((cb ^ swz(r1)) << 4) + ((i16 & 1) << 3);
   }
   // Called once per tile: hides v_base from loop-invariant code motion.
+  // With a 64-row q-block there are registers to spare and the compiler may keep all of them.
   auto v_addr_refresh = [&]() {
     v_cur = v_base;
-    asm volatile("" : "+v"(v_cur));
+    if constexpr (QBLK != 64) asm volatile("" : "+v"(v_cur));
   };
 
   // ---- building blocks --------------------------------------------------------------
@@ -416,6 +425,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
       const float new_sf = fmaxf(mr_sf, mloc_sf);
       const float alpha = (new_sf == kNegInf) ? 1.f : __builtin_amdgcn_exp2f(mr_sf - new_sf);
       mr_sf = new_sf;
+      base_eff = (new_sf == kNegInf) ? 0.f : new_sf;
       l_run *= alpha;
       if constexpr (HAS_V) {
 #pragma unroll
@@ -433,15 +443,15 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     for (int r = r0; r < r0 + cnt; r += 2) {
       const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[mb][r], p.sf, -base));
       const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[mb][r + 1], p.sf, -base));
-      l_run += e0;
-      l_run += e1;
+      l_tile = (mb == 0 && r == 0) ? e0 : l_tile + e0;
+      l_tile += e1;
       if constexpr (HAS_V) pb[2 * mb + (r >> 3)][(r & 7) >> 1] = pack_bf16(e0, e1);
     }
   };
   // Pin the softmax results where they are produced; otherwise the compiler sinks the
   // whole softmax to the first use of P and nothing overlaps the MFMAs.
   auto pin_softmax = [&]() {
-    asm volatile("" : "+v"(l_run));
+    asm volatile("" : "+v"(l_tile));
     if constexpr (HAS_V) {
 #pragma unroll
       for (int ks = 0; ks < 2 * NMB; ++ks)
@@ -450,9 +460,19 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     }
   };
   auto softmax_only = [&](f32x16 (&s)[NMB]) {
-    const float base = (mr_sf == kNegInf) ? 0.f : mr_sf;
 #pragma unroll
-    for (int mb = 0; mb < NMB; ++mb) softmax_chunk(s, base, mb, 0, 16);
+    for (int mb = 0; mb < NMB; ++mb) softmax_chunk(s, base_eff, mb, 0, 16);
+  };
+  // Closes the softmax of a tile: adds its sum to the denominator.  LAZY_MAX: first redoes
+  // the tile against a new reference if some row of the wave outgrew the old one.
+  auto softmax_close = [&](f32x16 (&s)[NMB]) {
+    if constexpr (LAZY_MAX) {
+      if (__any(!(l_tile <= kTrigger))) {
+        maybe_rescale(row_stats(s));
+        softmax_only(s);
+      }
+    }
+    l_run += l_tile;
   };
 
   // V^T operands of one 16-key step (PV group gi = 2mb + h), double-buffered over groups.
@@ -484,7 +504,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     constexpr bool WITH_SM = decltype(with_sm)::value;
     constexpr bool EARLY_V = decltype(early_v)::value;
     constexpr int EPM = 16 / NT;
-    const float base = (mr_sf == kNegInf) ? 0.f : mr_sf;
+    const float base = base_eff;
 #pragma unroll
     for (int mb = 0; mb < NMB; ++mb) {
       u32x4 ka[NT];
@@ -593,16 +613,18 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     const TileLoad tl_first = K_FIRST ? prepare_tile(it + NK, d_k, KN, false) : prepare_tile(it + 1, d_v, VN, true);
     qk_tile(std::true_type{}, std::integral_constant<bool, HAS_V>{}, KS * TILE, VS * TILE, s_b, s_a, &tl_first,
             K_FIRST ? has_kn : true);
+    softmax_close(s_a);
     mask_tile(it + 1, d_v, s_b);
     if constexpr (MODE != KV_TOKENS) idw[(KC + NK + 1) % 6] = tile_desc(it + NK + 1);
     float mloc_sf;
+    using stat_t = std::integral_constant<bool, !LAZY_MAX>;
     if constexpr (HAS_V) {
       const TileLoad tl_second = K_FIRST ? prepare_tile(it + 1, d_v, VN, true) : prepare_tile(it + NK, d_k, KN, false);
-      mloc_sf = pv_tile(std::true_type{}, std::true_type{}, VS * TILE, &tl_second, K_FIRST ? true : has_kn, s_b);
+      mloc_sf = pv_tile(std::true_type{}, stat_t{}, VS * TILE, &tl_second, K_FIRST ? true : has_kn, s_b);
     } else {
-      mloc_sf = pv_tile(std::true_type{}, std::true_type{}, 0, nullptr, false, s_b);
+      mloc_sf = pv_tile(std::true_type{}, stat_t{}, 0, nullptr, false, s_b);
     }
-    maybe_rescale(mloc_sf);
+    if constexpr (!LAZY_MAX) maybe_rescale(mloc_sf);
   };
   using I0 = std::integral_constant<int, 0>;
   using I1 = std::integral_constant<int, 1>;
@@ -652,7 +674,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
       }
     }
     // tail: softmax and P V of the last tile
-    if (it & 1) softmax_only(s_o); else softmax_only(s_e);
+    if (it & 1) { softmax_only(s_o); softmax_close(s_o); } else { softmax_only(s_e); softmax_close(s_e); }
     if constexpr (HAS_V) {
       wait_vmcnt<0>();
       __syncthreads();

@@ -146,6 +146,40 @@ def test_sp_attn_blocks_matches_oracle_and_token_path(dev, D, qblk, S):
 
 
 @pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("qblk", [64, 128])
+@pytest.mark.parametrize("growth", ["ramp", "jump"])
+def test_sp_attn_scores_that_outgrow_the_running_maximum(dev, D, qblk, growth):
+    """Keys whose scores grow along the list: the exponent reference has to move on later tiles
+    (a moderate ramp), also after a jump large enough to overflow exp2 against the old reference."""
+    print("case sp_attn growing scores", D, qblk, growth, flush=True)
+    B, H, S = 1, 2, 1024
+    q, k, v = wl.randn_qkv(B, H, S, D, seed=31)
+    kf = k.float()
+    blk = torch.arange(S) // 64
+    if growth == "ramp":
+        kf = kf * (1.0 + 0.75 * blk.float()).view(1, 1, S, 1)          # scores up to ~13x larger
+    else:
+        kf = kf * torch.where(blk >= 9, 600.0, 1.0).view(1, 1, S, 1)   # exponent jumps by thousands
+    k = kf.to(torch.bfloat16)
+    nk = S // 64
+    counts = np.full((B, H, orc.ceil_div(S, qblk)), nk)
+    bi, bc = wl.ragged_block_lists(B, H, S, qblk, 64, counts, seed=32)   # every block, ascending
+    qd, kd, vd, bid, bcd = to_dev(dev, q, k, v, bi, bc)
+    o = torch.full_like(qd, float("nan"))
+    lse = torch.full(q.shape[:3], float("nan"), device=dev)
+    capi.sp_attn_blocks(o, qd, kd, vd, bid, bcd, lse=lse, qblk=qblk)
+    tok, num = wl.blocks_to_tokens(bi, bc, S)
+    wo, wlse = orc.sp_attn(f32(q), f32(k), f32(v), tok.numpy(), num.numpy(), qblk=qblk)
+    assert_close_o(f32(o), wo, "growing scores, block path")
+    assert_close_stat(f32(lse), wlse, "lse", atol=1e-3)
+    o2, _ = _run_tokens(dev, q, k, v, tok, num, qblk)
+    assert_close_o(o2, wo, "growing scores, token path")
+    od = torch.full_like(qd, float("nan"))
+    capi.full_attn(od, qd, kd, vd)
+    assert_close_o(f32(od), wo, "growing scores, dense path")
+
+
+@pytest.mark.parametrize("D", [64, 128])
 @pytest.mark.parametrize("S,kv_len", [(512, 0), (1000, 0), (1000, 900), (130, 0)])
 def test_full_attn_and_stats(dev, D, S, kv_len):
     print("case full_attn", D, S, kv_len, flush=True)
