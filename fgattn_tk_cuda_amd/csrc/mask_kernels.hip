@@ -2,6 +2,8 @@
 //   booleanmask_128          - QK^T sweep -> per-(q-block, key) vote counts
 //   booleanmask_to_indexmask - vote mask -> ascending key-index lists (HBM-bound stream)
 //   all_index_mask           - identity lists
+#include <type_traits>
+
 #include "common.h"
 #include "dispatch.h"
 
@@ -15,11 +17,17 @@ namespace spattn {
 //   max_{r in W} (s[r,c] * sf - (max_q[r] * sf + log2 denom[r])) > log2 thresh.
 // Pad rows carry denom = -inf (include/maxq_denom.cuh:202-205) and never vote.
 //
-// One workgroup per q-block; the 128 x D query tile sits in LDS (16-byte chunks
-// XOR-swizzled by row) and is the A operand.  Each wave walks its own 32-key blocks: the
-// K^T operand goes HBM -> registers with no staging and no barrier, the accumulator of
-// lane (n, g) holds key n against 64 of the 128 query rows, and one exchange with lane
-// n^32 finishes the 8 votes of that key.  The vote count is stored, not accumulated.
+// One workgroup per q-block, each wave walks its own 32-key blocks.  Scores are S = Q K^T
+// with the query rows as the A operand - held in registers for d = 64 (each wave keeps
+// all 128 rows), read from an LDS copy of the tile for d = 128 - and the keys as the B
+// operand, loaded HBM -> registers one block ahead with no staging and no barrier.  The
+// accumulator of lane (n, g) holds key n against 64 of the 128 query rows.  The test is
+// rewritten once more as  s[r,c] - t[r] > 0  with the per-row constant
+// t[r] = (log2 thresh + max_q[r] sf + log2 denom[r]) / sf, and -t[r] is what the
+// accumulators start from: the matrix unit does the subtraction, the vector ALU only takes
+// the maximum of the 8 registers a lane holds of a 16-row group (v_max3) and compares it
+// with 0; one exchange with lane n^32 finishes the 8 votes of a key.  The vote count is
+// stored, not accumulated.
 // ------------------------------------------------------------------------------------
 template <int D>
 __global__ __launch_bounds__(256, 2) void booleanmask_kernel(int* __restrict__ mask, const float* __restrict__ max_q,
@@ -30,7 +38,9 @@ __global__ __launch_bounds__(256, 2) void booleanmask_kernel(int* __restrict__ m
                                                               int SB, float sf) {
   constexpr int NT = D / 16;
   constexpr int CPR = D / 8;
-  __shared__ __attribute__((aligned(16))) unsigned char qs[128 * D * 2];
+  constexpr bool Q_REGS = (D == 64);
+  __shared__ __attribute__((aligned(16))) unsigned char qs[Q_REGS ? 16 : 128 * D * 2];
+  __shared__ __attribute__((aligned(16))) float nthr_l[2][4][16];   // [g][mb][register]
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -45,79 +55,196 @@ __global__ __launch_bounds__(256, 2) void booleanmask_kernel(int* __restrict__ m
   const uint16_t* qh = q + head_off;
   const uint16_t* kh = k + head_off;
 
-  // Query tile -> LDS; rows past S are zero.
-  for (int ch = tid; ch < 128 * CPR; ch += 256) {
-    const int r = ch / CPR, c = ch % CPR;
-    const int row = qb * 128 + r;
-    u32x4 val = {0, 0, 0, 0};
-    if (row < S) val = *reinterpret_cast<const u32x4*>(qh + (size_t)row * D + 8 * c);
-    *reinterpret_cast<u32x4*>(qs + r * (D * 2) + ((c ^ (r & (CPR - 1))) << 4)) = val;
+  // Query rows; rows past S are zero.  In LDS the 16-byte chunk c of row r sits at
+  // c ^ swz(r), which spreads one chunk of 16 consecutive rows over all bank groups.
+  auto swz = [](int r) -> int { return ((r & 3) << 2) | ((r >> 2) & 3); };
+  u32x4 qa[Q_REGS ? 4 : 1][Q_REGS ? NT : 1];
+  if constexpr (Q_REGS) {
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb) {
+      const int row = qb * 128 + 32 * mb + ln;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const u32x4 z = {0, 0, 0, 0};
+        qa[mb][t] = (row < S) ? *reinterpret_cast<const u32x4*>(qh + (size_t)row * D + 16 * t + 8 * g) : z;
+      }
+    }
+  } else {
+    for (int ch = tid; ch < 128 * CPR; ch += 256) {
+      const int r = ch / CPR, c = ch % CPR;
+      const int row = qb * 128 + r;
+      u32x4 val = {0, 0, 0, 0};
+      if (row < S) val = *reinterpret_cast<const u32x4*>(qh + (size_t)row * D + 8 * c);
+      *reinterpret_cast<u32x4*>(qs + r * (D * 2) + ((c ^ swz(r)) << 4)) = val;
+    }
   }
 
-  // Per-row offsets; register 4j+i of block mb is query row 32mb + 8j + 4g + i.
-  float coff[4][16];
-#pragma unroll
-  for (int mb = 0; mb < 4; ++mb)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int row = qb * 128 + 32 * mb + 8 * (r >> 2) + 4 * g + (r & 3);
-      float c = __builtin_huge_valf();
-      if (row < S) {
-        const float mq = max_q[(size_t)bh * Sp + row];
-        const float dn = denom[(size_t)bh * Sp + row];
-        if (dn > 0.f) c = mq * sf + __log2f(dn);
-      }
-      coff[mb][r] = c;
+  // Minus the per-row thresholds on the raw score, as a table in LDS from which the
+  // accumulators are initialised; register 4j+i of block mb in lane half g is query row
+  // 32mb + 8j + 4g + i.  Pad rows and rows without keys get -inf and never vote.
+  const float inv_sf = 1.f / sf;
+  if (tid < 128) {
+    const int tg = tid >> 6, tmb = (tid >> 4) & 3, tr = tid & 15;
+    const int row = qb * 128 + 32 * tmb + 8 * (tr >> 2) + 4 * tg + (tr & 3);
+    float c = -__builtin_huge_valf();
+    if (row < S) {
+      const float mq = max_q[(size_t)bh * Sp + row];
+      const float dn = denom[(size_t)bh * Sp + row];
+      if (dn > 0.f) c = -(log2_thresh + (mq * sf + __log2f(dn))) * inv_sf;
     }
+    nthr_l[tg][tmb][tr] = c;
+  }
   __syncthreads();
 
   int* mrow = mask + ((size_t)bh * SB + qb) * mask_stride;
   const int nkb = (mask_stride + 31) >> 5;
 
+  // Keys past the end re-read the last key (their votes are never stored): the loads are
+  // unconditional, so the compiler can count them and let a block that was requested one
+  // step ahead stay in flight while the current one is multiplied.
   auto load_keys = [&](int kb, u32x4 (&kf)[NT]) {
-    const int key = kb * 32 + ln;
-    const bool ok = kb < nkb && key < kv_len;
+    int key = kb * 32 + ln;
+    key = key < kv_len ? key : kv_len - 1;
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      const u32x4 z = {0, 0, 0, 0};
-      kf[t] = ok ? *reinterpret_cast<const u32x4*>(kh + (size_t)key * D + 16 * t + 8 * g) : z;
+    for (int t = 0; t < NT; ++t) kf[t] = *reinterpret_cast<const u32x4*>(kh + (size_t)key * D + 16 * t + 8 * g);
+  };
+  // Bits 2mb, 2mb+1 of the result: does any of this lane's 8 rows of the two 16-row groups
+  // of block mb lie above its threshold.
+  // A float is > 0 exactly when its bit pattern, read as a signed integer, is > 0 (NaNs
+  // aside), and integer maxima need no NaN canonicalisation: v_max3_i32, 4 per 8 registers.
+  auto group_votes = [&](int mb, const f32x16& s) -> unsigned {
+    typedef __attribute__((ext_vector_type(16))) int i32x16;
+    const i32x16 si = __builtin_bit_cast(i32x16, s);
+    int w0 = si[0], w1 = si[8];
+#pragma unroll
+    for (int r = 1; r < 8; ++r) {
+      w0 = w0 > si[r] ? w0 : si[r];
+      w1 = w1 > si[8 + r] ? w1 : si[8 + r];
     }
+    return ((w0 > 0 ? 1u : 0u) << (2 * mb)) | ((w1 > 0 ? 1u : 0u) << (2 * mb + 1));
   };
 
-  u32x4 kf[NT], kn[NT];
-  load_keys(wave, kf);
-  for (int kb = wave; kb < nkb; kb += 4) {
-    load_keys(kb + 4, kn);
-    unsigned votes = 0;
-    if (kb * 32 < kv_len) {   // wave-uniform
+  // Software pipeline over half blocks (a pair of 32-row score blocks = 2 NT multiplies):
+  // while the matrix unit multiplies one pair, the vector ALU takes the maxima of the pair
+  // before it, a few vector instructions behind every multiply, so that a wave is an even
+  // mix of both at every point (two waves that alternate between a multiply-only and a
+  // vector-only phase fall into step and leave both units idle in turn).  Three accumulator
+  // sets rotate: multiplied now, reduced now, being initialised from the threshold table.
+  constexpr int NACC = Q_REGS ? 3 : 2;   // d = 128: registers for two sets only, the initialisation is then exposed
+  constexpr int NKS = Q_REGS ? 3 : 2;    // register sets of keys
+  f32x16 acc[NACC][2];
+  unsigned vhold = 0;
+  auto init_acc = [&](int p2, f32x16 (&dst)[2]) {
 #pragma unroll
-      for (int mb = 0; mb < 4; ++mb) {
-        f32x16 s;
+    for (int j = 0; j < 2; ++j) dst[j] = *reinterpret_cast<const f32x16*>(&nthr_l[g][2 * p2 + j][0]);
+  };
+  auto pair_scores = [&](int p2, const u32x4 (&kf)[NT], f32x16 (&a2)[2]) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s[r] = 0.f;
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int mb = 2 * p2 + j;
         const int qr = 32 * mb + ln;
-        const unsigned char* qrp = qs + qr * (D * 2);
-#pragma unroll
-        for (int t = 0; t < NT; ++t) {
-          const u32x4 a = *reinterpret_cast<const u32x4*>(qrp + (((2 * t + g) ^ (qr & (CPR - 1))) << 4));
-          s = mfma32(a, kf[t], s);
-        }
-        float w0 = -__builtin_huge_valf(), w1 = -__builtin_huge_valf();
-#pragma unroll
-        for (int r = 0; r < 8; ++r) {
-          w0 = fmaxf(w0, __builtin_fmaf(s[r], sf, -coff[mb][r]));
-          w1 = fmaxf(w1, __builtin_fmaf(s[8 + r], sf, -coff[mb][8 + r]));
-        }
-        votes |= (w0 > log2_thresh ? 1u : 0u) << (2 * mb);
-        votes |= (w1 > log2_thresh ? 1u : 0u) << (2 * mb + 1);
+        u32x4 a;
+        if constexpr (Q_REGS) a = qa[mb][t];
+        else a = *reinterpret_cast<const u32x4*>(qs + qr * (D * 2) + (((2 * t + g) ^ swz(qr)) << 4));
+        a2[j] = mfma32(a, kf[t], a2[j]);
       }
-    }
+  };
+  auto finish_block = [&](int kb, unsigned votes) {
     // A 16-row group is split over lanes n and n^32: it votes if either half does.
-    votes |= (unsigned)__shfl_xor((int)votes, 32, 64);
-    const int key = kb * 32 + ln;
-    if (g == 0 && key < mask_stride) mrow[key] = (key < kv_len) ? __popc(votes) : 0;
+    float lo_, hi_;
+    pair_values(__builtin_bit_cast(float, votes), lo_, hi_);   // v_permlane32_swap, no LDS
+    votes = __builtin_bit_cast(unsigned, lo_) | __builtin_bit_cast(unsigned, hi_);
+    const int key = kb * 32 + ln;   // negative for the block "before the first": nothing is stored
+    if (g == 0 && (unsigned)key < (unsigned)mask_stride) mrow[key] = (key < kv_len) ? __popc(votes) : 0;
+  };
+  // Half H: multiplies pair H&1 of block kb into acc[H % NACC], reduces the accumulators of
+  // the half before, initialises those of the half after.
+  auto half = [&](auto hc, int kb, const u32x4 (&kf)[NT]) {
+    constexpr int H = decltype(hc)::value;
+    constexpr int P = H & 1, A = H % NACC, AP = (H + NACC - 1) % NACC, AN = (H + 1) % NACC;
+    // with three sets the one for the next half is free now: its initial values travel from
+    // LDS while this half is multiplied
+    if constexpr (NACC == 3) init_acc(1 - P, acc[AN]);
+    pair_scores(P, kf, acc[A]);
+    const unsigned v = group_votes(2 * (1 - P), acc[AP][0]) | group_votes(2 * (1 - P) + 1, acc[AP][1]);
 #pragma unroll
-    for (int t = 0; t < NT; ++t) kf[t] = kn[t];
+    for (int i = 0; i < 2 * NT; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, (NT == 4) ? 3 : 2, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (NACC != 3) init_acc(1 - P, acc[AN]);
+    if constexpr (P == 0) finish_block(kb - 4, vhold | v);   // pair 1 of the block before
+    else vhold = v;                                          // pair 0 of this block
+  };
+  // After the last block (its second half went into acc[A]): reduce it and store.
+  auto drain = [&](auto ac, int kb) {
+    constexpr int A = decltype(ac)::value;
+    finish_block(kb, vhold | group_votes(2, acc[A][0]) | group_votes(3, acc[A][1]));
+  };
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  using I2 = std::integral_constant<int, 2>;
+  using I3 = std::integral_constant<int, 3>;
+  using I4 = std::integral_constant<int, 4>;
+  using I5 = std::integral_constant<int, 5>;
+
+  // Key sets rotate without copies; a set is requested NKS-1 whole blocks before it is
+  // multiplied (a block is 4 NT multiplies, far shorter than a trip to L2).  The main loop
+  // runs whole rotations without side exits; at most NKS-1 blocks remain after it.
+  int kb = wave;
+  init_acc(0, acc[0]);
+  init_acc(1, acc[NACC - 1]);   // reduced by the very first half; its votes go nowhere
+  if constexpr (NKS == 3) {
+    u32x4 k0[NT], k1[NT], k2[NT];
+    load_keys(kb, k0);
+    load_keys(kb + 4, k1);
+    while (kb + 8 < nkb) {
+      load_keys(kb + 8, k2);
+      half(I0{}, kb, k0);
+      half(I1{}, kb, k0);
+      load_keys(kb + 12, k0);
+      half(I2{}, kb + 4, k1);
+      half(I3{}, kb + 4, k1);
+      load_keys(kb + 16, k1);
+      half(I4{}, kb + 8, k2);
+      half(I5{}, kb + 8, k2);
+      kb += 12;
+    }
+    if (kb < nkb) {
+      half(I0{}, kb, k0);
+      half(I1{}, kb, k0);
+      if (kb + 4 < nkb) {
+        half(I2{}, kb + 4, k1);
+        half(I3{}, kb + 4, k1);
+        drain(std::integral_constant<int, 3 % NACC>{}, kb + 4);
+      } else {
+        drain(std::integral_constant<int, 1 % NACC>{}, kb);
+      }
+    } else {
+      drain(std::integral_constant<int, 5 % NACC>{}, kb - 4);
+    }
+  } else {
+    u32x4 k0[NT], k1[NT];
+    load_keys(kb, k0);
+    while (kb + 4 < nkb) {
+      load_keys(kb + 4, k1);
+      half(I0{}, kb, k0);
+      half(I1{}, kb, k0);
+      load_keys(kb + 8, k0);
+      half(I0{}, kb + 4, k1);
+      half(I1{}, kb + 4, k1);
+      kb += 8;
+    }
+    if (kb < nkb) {
+      half(I0{}, kb, k0);
+      half(I1{}, kb, k0);
+      drain(I1{}, kb);
+    } else {
+      drain(I1{}, kb - 4);
+    }
   }
 }
 
