@@ -35,7 +35,7 @@ PEAK_HBM_GBPS = 8000.0
 # file (--only sparse / --only compact), scaled by what the same counters read for the plain
 # 1 GiB copy of --only copy (FETCH_SIZE x2.0, WRITE_SIZE x1.0).  Text summaries of those runs
 # sit in profiles/counters_*.txt; they are measured offline, not in this process.
-TRAFFIC_SPARSE_BYTES = 5.36e9 + 0.675e9     # fetch + write of attn_fwd_kernel<128,64,KV_BLOCKS>
+TRAFFIC_SPARSE_BYTES = 4.746e9 + 0.2726e9   # rocprofv3 FETCH_SIZE x2.0 + WRITE_SIZE x1.0, see profiles/
 TRAFFIC_COMPACT_BYTES = 805.4e6 + 64.5e6    # fetch + write of compact_kernel
 
 
