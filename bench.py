@@ -117,6 +117,27 @@ def bench_compaction(dev, steps, warmup, seed=0):
     return dict(ms=ms, bytes=nbytes, kept=kept, shape=[B, H, SB, ms_])
 
 
+def bench_packed(dev, steps, warmup, seed=0):
+    """The bit-packed mask cache at the same mask: pack_mask (int32 votes -> bits) and
+    packedmask_to_indexmask (bits -> index lists, the fused unpack + compaction)."""
+    c = wl.CONFIGS["cfg4_threshold_padded"]
+    B, H, S = c["B"], c["H"], c["S"]
+    ms_ = 128 * wl.ceil_div(S, 128)
+    SB = ms_ // 128
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    mask = (torch.rand((B, H, SB, ms_), device=dev, generator=g) < c["keep"]).to(torch.int32)
+    packed = torch.empty((B, H, SB, ms_ // 8), dtype=torch.uint8, device=dev)
+    kvi = torch.full((B, H, SB, ms_), ms_, dtype=torch.int32, device=dev)
+    kvn = torch.zeros((B, H, SB), dtype=torch.int32, device=dev)
+    ms_pack, _ = time_steps(lambda: capi.pack_mask(packed, mask), steps, warmup)
+    ms_idx, _ = time_steps(lambda: capi.packedmask_to_indexmask(kvi, kvn, packed, S), steps, warmup)
+    kept = int(kvn.sum().item())
+    rows = B * H * SB
+    return dict(ms_pack=ms_pack, bytes_pack=4.0 * rows * ms_ + rows * ms_ / 8.0,
+                ms_index=ms_idx, bytes_index=rows * ms_ / 8.0 + 4.0 * kept + 4.0 * rows, kept=kept)
+
+
 def bench_copy(dev, steps, warmup, seed=0):
     """A plain 1 GiB device-to-device copy: the known-size kernel that the FETCH_SIZE /
     WRITE_SIZE counters of the other kernels are scaled by."""
@@ -196,7 +217,7 @@ def main(argv=None) -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-extras", action="store_true", help="only the headline kernel")
-    ap.add_argument("--only", default="", help="run one leg only: sparse|compact|dense|sweeps|copy (no JSON contract)")
+    ap.add_argument("--only", default="", help="run one leg only: sparse|compact|dense|sweeps|copy|packed (no JSON contract)")
     args = ap.parse_args(argv)
     if args.gpus != 1:
         print("bench.py: this library is single-GPU; run with --gpus 1 (got %d)" % args.gpus, file=sys.stderr)
@@ -210,7 +231,7 @@ def main(argv=None) -> int:
 
     if args.only:
         fn = {"sparse": bench_sparse, "compact": bench_compaction, "dense": bench_dense, "sweeps": bench_sweeps,
-              "copy": bench_copy}[args.only]
+              "copy": bench_copy, "packed": bench_packed}[args.only]
         r = fn(dev, args.steps, args.warmup)
         r.pop("tensors", None)
         print(json.dumps(r))
@@ -239,6 +260,14 @@ def main(argv=None) -> int:
                             "roofline": {"bound": "hbm", "achieved": gbps, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                                          "frac": gbps / PEAK_HBM_GBPS, "traffic": TRAFFIC_COMPACT_BYTES,
                                          "traffic_unit": "bytes", "algorithmic_bytes": cp["bytes"]}}
+        pk = bench_packed(dev, args.steps, args.warmup)
+        out["mask_cache"] = {
+            "workload": "same mask, bit-packed (1 bit per key)",
+            "pack_mask_ms": pk["ms_pack"], "pack_mask_gbps": pk["bytes_pack"] / pk["ms_pack"] / 1e6,
+            "pack_mask_hbm_frac": pk["bytes_pack"] / pk["ms_pack"] / 1e6 / PEAK_HBM_GBPS,
+            "packedmask_to_indexmask_ms": pk["ms_index"], "packedmask_to_indexmask_gbps": pk["bytes_index"] / pk["ms_index"] / 1e6,
+            "packedmask_to_indexmask_hbm_frac": pk["bytes_index"] / pk["ms_index"] / 1e6 / PEAK_HBM_GBPS,
+            "algorithmic_bytes": [pk["bytes_pack"], pk["bytes_index"]]}
         dn = bench_dense(dev, args.steps, args.warmup)
         out["dense_full_attn"] = {"workload": "cfg2: B=4 H=16 N=4096 d=64", "ms": dn["ms"],
                                   "tflops": dn["flops"] / (dn["ms"] * 1e-3) / 1e12,

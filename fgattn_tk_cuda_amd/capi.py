@@ -35,6 +35,8 @@ _SIGNATURES = {
     "spattn_maxq_denom": (_c_int, [_c_void_p] * 4 + [_c_int] * 5 + [_c_float, _c_void_p]),
     "spattn_booleanmask_128": (_c_int, [_c_void_p, _c_float, _c_int] + [_c_void_p] * 4 + [_c_int] * 5 + [_c_float, _c_void_p]),
     "spattn_booleanmask_to_indexmask": (_c_int, [_c_void_p] * 3 + [_c_int] * 5 + [_c_void_p]),
+    "spattn_pack_mask": (_c_int, [_c_void_p] * 2 + [_c_int] * 4 + [_c_void_p]),
+    "spattn_packedmask_to_indexmask": (_c_int, [_c_void_p] * 3 + [_c_int] * 5 + [_c_void_p]),
     "spattn_last_status": (_c_int, []),
     "spattn_status_string": (ctypes.c_char_p, [_c_int]),
     "spattn_version": (_c_int, []),
@@ -174,6 +176,28 @@ def booleanmask_to_indexmask(kv_indices, kv_num_indices, booleanmask, seq, *, st
         raise ValueError("kv_indices / kv_num_indices do not match booleanmask")
     _check(load().spattn_booleanmask_to_indexmask(_ptr(kv_indices, i32), _ptr(kv_num_indices, i32),
                                                   _ptr(booleanmask, i32), B, H, int(seq), SB, MS, _stream(stream)))
+
+
+def pack_mask(packed, booleanmask, *, stream=None):
+    """packed: uint8 [B,H,SB,mask_stride/8]; bit (c & 7) of byte c >> 3 is set where booleanmask[..., c] > 0."""
+    if booleanmask.dim() != 4:
+        raise ValueError("booleanmask must be [B,H,SB,mask_stride]")
+    B, H, SB, MS = (int(x) for x in booleanmask.shape)
+    if tuple(packed.shape) != (B, H, SB, MS // 8) or MS % 8:
+        raise ValueError("packed must be uint8 [B,H,SB,mask_stride/8]")
+    _check(load().spattn_pack_mask(_ptr(packed, torch.uint8), _ptr(booleanmask, i32), B, H, SB, MS, _stream(stream)))
+
+
+def packedmask_to_indexmask(kv_indices, kv_num_indices, packed, seq, *, stream=None):
+    """Index lists straight from a bit-packed mask (uint8 [B,H,SB,mask_stride/8])."""
+    if packed.dim() != 4:
+        raise ValueError("packed must be [B,H,SB,mask_stride/8]")
+    B, H, SB, MB = (int(x) for x in packed.shape)
+    MS = MB * 8
+    if tuple(kv_indices.shape) != (B, H, SB, MS) or kv_num_indices.numel() != B * H * SB:
+        raise ValueError("kv_indices / kv_num_indices do not match the packed mask")
+    _check(load().spattn_packedmask_to_indexmask(_ptr(kv_indices, i32), _ptr(kv_num_indices, i32),
+                                                 _ptr(packed, torch.uint8), B, H, int(seq), SB, MS, _stream(stream)))
 
 
 def infer_qblk(seq: int, seqblocks: int) -> int:

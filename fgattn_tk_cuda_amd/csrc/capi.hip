@@ -143,6 +143,25 @@ int spattn_booleanmask_to_indexmask(int* kv_indices, int* num_kv_indices, const 
                                       as_stream(stream)));
 }
 
+int spattn_pack_mask(void* packed, const int* booleanmask, int B, int H, int seqblocks, int mask_stride, void* stream) {
+  if (!packed || !booleanmask) return done(SPATTN_ERR_NULL);
+  if (B <= 0 || H <= 0 || seqblocks <= 0) return done(SPATTN_ERR_SHAPE);
+  if (mask_stride <= 0 || mask_stride % 128 != 0) return done(SPATTN_ERR_STRIDE);
+  if (misaligned(packed) || misaligned(booleanmask)) return done(SPATTN_ERR_ALIGN);
+  return from_hip(spattn::run_pack_mask(static_cast<uint32_t*>(packed), booleanmask, B * H * seqblocks, mask_stride,
+                                        as_stream(stream)));
+}
+
+int spattn_packedmask_to_indexmask(int* kv_indices, int* num_kv_indices, const void* packed, int B, int H, int seq,
+                                   int seqblocks, int mask_stride, void* stream) {
+  if (!kv_indices || !num_kv_indices || !packed) return done(SPATTN_ERR_NULL);
+  if (B <= 0 || H <= 0 || seqblocks <= 0 || seq < 0) return done(SPATTN_ERR_SHAPE);
+  if (mask_stride <= 0 || mask_stride % 128 != 0) return done(SPATTN_ERR_STRIDE);
+  if (misaligned(kv_indices) || misaligned(packed)) return done(SPATTN_ERR_ALIGN);
+  return from_hip(spattn::run_packed_to_indexmask(kv_indices, num_kv_indices, static_cast<const uint32_t*>(packed),
+                                                  B * H * seqblocks, mask_stride, seq, as_stream(stream)));
+}
+
 // ---- the reference's binding surface: default stream, default scale, q-block 128 ----
 
 void attn_fwd_wg_impl(void* o, void* q, void* k, void* v, int batch, int heads, int seq, int D) {

@@ -17,4 +17,9 @@ hipError_t run_compact(int* kv_indices, int* kv_num, const int* mask, int rows, 
                        hipStream_t stream);
 hipError_t run_all_index(int* kv_indices, int* kv_num, int rows, int mask_stride, int seq, hipStream_t stream);
 
+// bitmask_kernels.hip
+hipError_t run_pack_mask(uint32_t* packed, const int* mask, int rows, int mask_stride, hipStream_t stream);
+hipError_t run_packed_to_indexmask(int* kv_indices, int* kv_num, const uint32_t* packed, int rows, int mask_stride,
+                                   int kv_len, hipStream_t stream);
+
 }  // namespace spattn

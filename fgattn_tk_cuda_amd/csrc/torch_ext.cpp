@@ -160,12 +160,48 @@ void booleanmask_to_indexmask(torch::Tensor kv_indices, torch::Tensor kv_numindi
                "booleanmask_to_indexmask");
 }
 
+// Two operators beyond the reference's seven, for its bit-packed mask cache
+// (python/spattn/mask_utils.py:74-98,421-439): the cache's torch-level pack / unpack become
+// one kernel each way.
+void pack_mask(torch::Tensor packed, torch::Tensor booleanmask) {
+  TORCH_CHECK(booleanmask.is_cuda() && booleanmask.scalar_type() == at::kInt && booleanmask.is_contiguous() &&
+                  booleanmask.dim() == 4,
+              "booleanmask must be a contiguous int32 device tensor [B,H,SB,mask_stride]");
+  check_aux(packed, "packed", at::kByte, booleanmask);
+  TORCH_CHECK(packed.dim() == 4 && packed.size(0) == booleanmask.size(0) && packed.size(1) == booleanmask.size(1) &&
+                  packed.size(2) == booleanmask.size(2) && packed.size(3) * 8 == booleanmask.size(3),
+              "packed must be uint8 [B,H,SB,mask_stride/8]");
+  const DeviceGuard guard(booleanmask.device());
+  check_status(spattn_pack_mask(packed.data_ptr(), booleanmask.data_ptr<int>(), (int)booleanmask.size(0),
+                                (int)booleanmask.size(1), (int)booleanmask.size(2), (int)booleanmask.size(3), cur_stream()),
+               "pack_mask");
+}
+
+void packedmask_to_indexmask(torch::Tensor kv_indices, torch::Tensor kv_numindices, torch::Tensor packed, int64_t seq) {
+  TORCH_CHECK(packed.is_cuda() && packed.scalar_type() == at::kByte && packed.is_contiguous() && packed.dim() == 4,
+              "packed must be a contiguous uint8 device tensor [B,H,SB,mask_stride/8]");
+  check_aux(kv_indices, "kv_indices", at::kInt, packed);
+  check_aux(kv_numindices, "kv_numindices", at::kInt, packed);
+  TORCH_CHECK(kv_indices.dim() == 4 && kv_indices.size(0) == packed.size(0) && kv_indices.size(1) == packed.size(1) &&
+                  kv_indices.size(2) == packed.size(2) && kv_indices.size(3) == packed.size(3) * 8,
+              "kv_indices must be [B,H,SB,mask_stride]");
+  TORCH_CHECK(kv_numindices.numel() == packed.size(0) * packed.size(1) * packed.size(2),
+              "kv_numindices must have B*H*SB entries");
+  TORCH_CHECK(seq >= 0, "seq must not be negative");
+  const DeviceGuard guard(packed.device());
+  check_status(spattn_packedmask_to_indexmask(kv_indices.data_ptr<int>(), kv_numindices.data_ptr<int>(), packed.data_ptr(),
+                                              (int)packed.size(0), (int)packed.size(1), (int)seq, (int)packed.size(2),
+                                              (int)packed.size(3) * 8, cur_stream()),
+               "packedmask_to_indexmask");
+}
+
 // Meta kernels: shapes only, nothing to compute (all ops mutate their arguments in place).
 void noop4(torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor) {}
 void noop_all_index(torch::Tensor, torch::Tensor, int64_t, int64_t, int64_t, int64_t) {}
 void noop6(torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor) {}
 void noop_mask(torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, double) {}
 void noop_b2i(torch::Tensor, torch::Tensor, torch::Tensor, int64_t) {}
+void noop2(torch::Tensor, torch::Tensor) {}
 
 TORCH_LIBRARY_FRAGMENT(cuda_attn, m) {
   m.def("full_attn(Tensor(a!) o, Tensor q, Tensor k, Tensor v) -> ()");
@@ -175,6 +211,8 @@ TORCH_LIBRARY_FRAGMENT(cuda_attn, m) {
   m.def("maxq_denom(Tensor(a!) o_max_q, Tensor(b!) o_denom, Tensor q, Tensor k) -> ()");
   m.def("booleanmask_128(Tensor(a!) booleanmask, Tensor o_max_q, Tensor o_denom, Tensor q, Tensor k, float threshold) -> ()");
   m.def("booleanmask_to_indexmask(Tensor(a!) kv_indices, Tensor(b!) kv_numindices, Tensor booleanmask, int seq) -> ()");
+  m.def("pack_mask(Tensor(a!) packed, Tensor booleanmask) -> ()");
+  m.def("packedmask_to_indexmask(Tensor(a!) kv_indices, Tensor(b!) kv_numindices, Tensor packed, int seq) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(cuda_attn, Meta, m) {
@@ -185,6 +223,8 @@ TORCH_LIBRARY_IMPL(cuda_attn, Meta, m) {
   m.impl("maxq_denom", noop4);
   m.impl("booleanmask_128", noop_mask);
   m.impl("booleanmask_to_indexmask", noop_b2i);
+  m.impl("pack_mask", noop2);
+  m.impl("packedmask_to_indexmask", noop_b2i);
 }
 
 // The CUDA dispatch key serves HIP tensors on PyTorch-ROCm.
@@ -196,6 +236,8 @@ TORCH_LIBRARY_IMPL(cuda_attn, CUDA, m) {
   m.impl("maxq_denom", maxq_denom);
   m.impl("booleanmask_128", booleanmask_128);
   m.impl("booleanmask_to_indexmask", booleanmask_to_indexmask);
+  m.impl("pack_mask", pack_mask);
+  m.impl("packedmask_to_indexmask", packedmask_to_indexmask);
 }
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -206,4 +248,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("booleanmask_128", &booleanmask_128, "booleanmask_128");
   m.def("booleanmask_to_indexmask", &booleanmask_to_indexmask, "booleanmask_to_indexmask");
   m.def("fullattn_maxq_denom", &fullattn_maxq_denom, "fullattn_maxq_denom");
+  m.def("pack_mask", &pack_mask, "pack_mask");
+  m.def("packedmask_to_indexmask", &packedmask_to_indexmask, "packedmask_to_indexmask");
 }

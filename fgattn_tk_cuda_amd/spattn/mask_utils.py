@@ -72,14 +72,21 @@ class BitMaskCache:
 
 
 class CompressedBitMaskCache(BitMaskCache):
-    """Stores the mask bit-packed (8 keys per byte, least significant bit first)."""
+    """Stores the mask bit-packed (8 keys per byte, least significant bit first).  On the device
+    both directions are single kernels: the vote mask is packed without a boolean copy, and a
+    reuse goes from the bits to the index lists without materialising the unpacked mask."""
 
     def get_mask_from_cache(self, layer):
         packed, seq_len = self.cache[layer]
+        if packed.is_cuda and packed.dim() == 4:
+            return packedmask_to_indexmask_cuda(packed, seq_len)
         return bitmask_to_indexmask_cuda(unpack(packed).to(torch.int32), seq_len)
 
     def update_cache(self, layer, bitmask, seq_len):
-        self.cache[layer] = (pack(bitmask > 0), seq_len)
+        if bitmask.is_cuda and bitmask.dim() == 4 and bitmask.dtype == torch.int32 and bitmask.shape[-1] % 128 == 0:
+            self.cache[layer] = (pack_votes_cuda(bitmask), seq_len)
+        else:
+            self.cache[layer] = (pack(bitmask > 0), seq_len)
 
 
 # ----------------------------------------------------------------------------------
@@ -207,6 +214,28 @@ def bitmask_to_indexmask_cuda(booleanmask, seq=None):
     kv_indices = torch.full((B, H, SB, MS), MS, dtype=torch.int32, device=booleanmask.device)
     num_kv_indices = torch.zeros((B, H, SB), dtype=torch.int32, device=booleanmask.device)
     spattn_interface.booleanmask_to_indexmask(kv_indices, num_kv_indices, booleanmask.to(torch.int32).contiguous(), seq)
+    return kv_indices, num_kv_indices
+
+
+def pack_votes_cuda(booleanmask):
+    """uint8 [B,H,SB,mask_stride/8]: bit (c & 7) of byte c >> 3 set where the int32 vote mask is > 0;
+    equals ``pack(booleanmask > 0)``."""
+    B, H, SB, MS = booleanmask.shape
+    packed = torch.empty((B, H, SB, MS // 8), dtype=torch.uint8, device=booleanmask.device)
+    spattn_interface.pack_mask(packed, booleanmask.contiguous())
+    return packed
+
+
+def packedmask_to_indexmask_cuda(packed, seq=None):
+    """Index lists and counts straight from a bit-packed mask; equals
+    ``bitmask_to_indexmask_cuda(unpack(packed), seq)``."""
+    B, H, SB, MB = packed.shape
+    MS = MB * 8
+    if seq is None:
+        seq = MS
+    kv_indices = torch.full((B, H, SB, MS), MS, dtype=torch.int32, device=packed.device)
+    num_kv_indices = torch.zeros((B, H, SB), dtype=torch.int32, device=packed.device)
+    spattn_interface.packedmask_to_indexmask(kv_indices, num_kv_indices, packed.contiguous(), seq)
     return kv_indices, num_kv_indices
 
 

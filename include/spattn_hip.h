@@ -108,6 +108,19 @@ int spattn_booleanmask_128(int* booleanmask, float threshold, int mask_stride, c
 int spattn_booleanmask_to_indexmask(int* kv_indices, int* num_kv_indices, const int* booleanmask, int batch, int heads,
                                     int seq, int seqblocks, int mask_stride, void* stream);
 
+/* Bit-packed masks for the mask cache: one bit per key, least significant bit first, rows of
+ * mask_stride / 8 bytes -- the layout of `pack` (python/spattn/mask_utils.py:421-430).
+ * spattn_pack_mask sets a bit where the int32 vote mask is > 0 (what
+ * CompressedBitMaskCache.update_cache stores, python/spattn/mask_utils.py:92-98);
+ * spattn_packedmask_to_indexmask is the fused form of `unpack` followed by
+ * booleanmask_to_indexmask (CompressedBitMaskCache.get_mask_from_cache,
+ * python/spattn/mask_utils.py:86-90): ascending keys c < seq whose bit is set, then the
+ * caller's fill; exact counts.  `packed` holds batch*heads*seqblocks*mask_stride/8 bytes. */
+int spattn_pack_mask(void* packed, const int* booleanmask, int batch, int heads, int seqblocks, int mask_stride,
+                     void* stream);
+int spattn_packedmask_to_indexmask(int* kv_indices, int* num_kv_indices, const void* packed, int batch, int heads,
+                                   int seq, int seqblocks, int mask_stride, void* stream);
+
 /* Status of the most recent call on this host thread, and its text. */
 int spattn_last_status(void);
 const char* spattn_status_string(int status);

@@ -276,3 +276,23 @@ def block_mask_from_votes(votes, seq: int, kvblk: int = 64):
     if pad:
         m = np.concatenate([m, np.zeros((B, H, SB, pad), bool)], axis=-1)
     return m.reshape(B, H, SB, nb, kvblk).any(axis=-1)
+
+
+def pack_mask(mask):
+    """Bit-packed form of a vote mask: bit (c & 7) of byte c >> 3 is set where mask[..., c] > 0
+    (python/spattn/mask_utils.py:421-430, `pack`: 8 booleans per byte, least significant bit first).
+    Pinned by numpy.packbits(bitorder='little'), a library routine, and by the round trip below."""
+    mask = np.asarray(mask)
+    assert mask.shape[-1] % 8 == 0
+    return np.packbits(mask > 0, axis=-1, bitorder="little")
+
+
+def unpack_mask(packed):
+    """Inverse of pack_mask as booleans (python/spattn/mask_utils.py:432-439, `unpack`)."""
+    return np.unpackbits(np.asarray(packed, np.uint8), axis=-1, bitorder="little").astype(bool)
+
+
+def packedmask_to_indexmask(packed, seq, fill=None):
+    """unpack followed by booleanmask_to_indexmask: what CompressedBitMaskCache.get_mask_from_cache
+    computes (python/spattn/mask_utils.py:86-90)."""
+    return booleanmask_to_indexmask(unpack_mask(packed).astype(np.int32), seq, fill=fill)

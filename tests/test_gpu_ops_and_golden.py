@@ -103,6 +103,18 @@ def test_operator_extension_on_device(dev):
     idx_d, num_d = mu.qk_indexmask_cuda(q, k, thr)
     idx_r, num_r = mu.bitmask_to_indexmask(mu.qk_bitmask_cuda(q, k, thr))
     assert torch.equal(idx_d, idx_r) and torch.equal(num_d, num_r)
+    # the bit-packed cache path: one kernel each way equals the torch-level pack / unpack + compaction
+    votes = mu.qk_bitmask_from_maxq_denom_cuda(mx2, dn2, q, k, thr)
+    packed = mu.pack_votes_cuda(votes)
+    assert torch.equal(packed, mu.pack(votes > 0))
+    idx_p, num_p = mu.packedmask_to_indexmask_cuda(packed, S)
+    idx_u, num_u = mu.bitmask_to_indexmask_cuda(mu.unpack(packed).to(torch.int32), S)
+    assert torch.equal(idx_p, idx_u) and torch.equal(num_p, num_u)
+    cache = mu.CompressedBitMaskCache([0])
+    cache.update_cache(3, votes, S)
+    assert cache.cache[3][0].dtype == torch.uint8 and cache.cache[3][0].shape[-1] * 8 == votes.shape[-1]
+    idx_c, num_c = cache.get_mask_from_cache(3)
+    assert torch.equal(idx_c, idx_u) and torch.equal(num_c, num_u)
     # errors are raised, not swallowed
     with pytest.raises(RuntimeError):
         ops.full_attn(o, q.float(), k, v)

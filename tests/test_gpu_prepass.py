@@ -61,6 +61,32 @@ def test_compaction_bit_exact(dev, SB, ms, seq, density):
     assert np.array_equal(kvi.cpu().numpy(), wi)
 
 
+@pytest.mark.parametrize("SB,ms,seq,density", [(3, 128, 128, 0.3), (2, 1024, 1000, 0.08), (2, 8192 + 256, 8192 + 200, 0.08),
+                                               (1, 16384, 16384, 1.0), (2, 2048, 0, 0.5), (2, 4096, 4096, 0.0),
+                                               (1, 32768, 32760, 0.5)])
+def test_packed_mask_round_trip_bit_exact(dev, SB, ms, seq, density):
+    """pack_mask == numpy.packbits (LSB first); packedmask_to_indexmask == unpack + compaction, bit for bit;
+    and on the device the packed path gives exactly what the int32 path gives."""
+    print("case packed mask", SB, ms, seq, density, flush=True)
+    B, H = 2, 2
+    rng = np.random.default_rng(70)
+    mask = (rng.random((B, H, SB, ms)) < density).astype(np.int32) * rng.integers(1, 9, size=(B, H, SB, ms), dtype=np.int32)
+    md = torch.from_numpy(mask).to(dev)
+    packed = torch.full((B, H, SB, ms // 8), 0xA5, dtype=torch.uint8, device=dev)
+    capi.pack_mask(packed, md)
+    assert np.array_equal(packed.cpu().numpy(), orc.pack_mask(mask))
+    kvi = torch.full((B, H, SB, ms), ms, dtype=torch.int32, device=dev)
+    kvn = torch.full((B, H, SB), -1, dtype=torch.int32, device=dev)
+    capi.packedmask_to_indexmask(kvi, kvn, packed, seq)
+    wi, wn = orc.packedmask_to_indexmask(orc.pack_mask(mask), seq)
+    assert np.array_equal(kvn.cpu().numpy(), wn)
+    assert np.array_equal(kvi.cpu().numpy(), wi)
+    kvi2 = torch.full((B, H, SB, ms), ms, dtype=torch.int32, device=dev)
+    kvn2 = torch.full((B, H, SB), -1, dtype=torch.int32, device=dev)
+    capi.booleanmask_to_indexmask(kvi2, kvn2, md, seq)
+    assert torch.equal(kvi, kvi2) and torch.equal(kvn, kvn2)
+
+
 def test_all_index_mask(dev):
     print("case all_index_mask", flush=True)
     B, H, SB, S, ms = 2, 3, 5, 600, 640

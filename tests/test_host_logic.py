@@ -68,6 +68,7 @@ def test_torch_mask_helpers_match_oracle():
     b = torch.from_numpy(rng.random((2, 3, 64)) < 0.5)
     assert torch.equal(mu.unpack(mu.pack(b)), b)
     assert mu.pack(torch.tensor([[True, False, False, False, False, False, False, True]])).item() == 129
+    assert np.array_equal(mu.pack(b).numpy(), orc.pack_mask(b.numpy()))
     a = torch.rand(300, 8)
     assert torch.equal(mu.attnmapor(a, 128)[2], a[256:].max(0).values)
     assert torch.equal(mu.attnmapand(a, 128)[0], a[:128].min(0).values)

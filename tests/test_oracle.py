@@ -204,3 +204,24 @@ def test_bf16_round():
     x = np.array([1.0, 1.00390625, 1.01171875, -3.1415926, 1e-30, 65504.0], np.float32)
     want = torch.from_numpy(x).to(torch.bfloat16).float().numpy()
     assert np.array_equal(orc.bf16_round(x), want)
+
+
+def test_pack_mask_matches_library_and_round_trips():
+    """pack: 8 keys per byte, least significant bit first (numpy.packbits little); unpack inverts it
+    (the reference's own round-trip test, python/test/spattn/test_mask_utils.py:86-97); the byte value of a
+    hand-made pattern; the fused unpack+compaction equals compaction of the unpacked mask."""
+    rng = np.random.default_rng(3)
+    mask = (rng.random((1, 2, 3, 256)) < 0.2).astype(np.int32) * 5
+    packed = orc.pack_mask(mask)
+    assert packed.dtype == np.uint8 and packed.shape == (1, 2, 3, 32)
+    assert np.array_equal(orc.unpack_mask(packed), mask > 0)
+    one = np.zeros((1, 1, 1, 8), np.int32)
+    one[..., 0] = 1
+    one[..., 7] = 3
+    assert orc.pack_mask(one).item() == 129
+    # brute force, bit by bit
+    for c in range(256):
+        assert ((packed[0, 1, 2, c >> 3] >> (c & 7)) & 1) == (mask[0, 1, 2, c] > 0)
+    wi, wn = orc.packedmask_to_indexmask(packed, 200)
+    ri, rn = orc.booleanmask_to_indexmask(mask, 200)
+    assert np.array_equal(wi, ri) and np.array_equal(wn, rn)
