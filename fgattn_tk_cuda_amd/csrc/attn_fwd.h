@@ -46,8 +46,6 @@
 namespace spattn {
 
 typedef __attribute__((ext_vector_type(4))) short s16x4;
-#define SPATTN_LDS __attribute__((address_space(3)))
-typedef SPATTN_LDS const unsigned char* lds_cptr;
 
 template <int D, int MODE, bool HAS_V>
 struct AttnCfg {
@@ -65,28 +63,6 @@ struct AttnCfg {
   static constexpr int kRowsPerLoad = 1024 / (D * 2);         // rows one wave-wide 1 KB load covers
   static constexpr int kLoadsPerTile = kTileBytes / 1024 / 4;   // per wave
 };
-
-// One wave-wide HBM -> LDS copy: lane l's 16 bytes land at lds_base + 16 l.
-// Written as asm on purpose: the compiler does not count this load in its own vmcnt
-// bookkeeping (with the builtin it drains every outstanding load before each LDS read),
-// so the waits are placed by hand.
-__device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(gptr) : "memory");
-}
-// Same with a wave-uniform base pointer and a 32-bit per-lane byte offset.
-// The base goes through readfirstlane: under scalar-register pressure the compiler may keep
-// a uniform pointer in vector registers, which the "s" constraint alone does not undo.
-__device__ __forceinline__ void dma16(const void* sbase, uint32_t voff, uint32_t lds_base) {
-  const uint64_t b = (uint64_t)(uintptr_t)sbase;
-  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)b);
-  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
-  const uint64_t sb = ((uint64_t)hi << 32) | lo;
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(voff), "s"(sb) : "memory");
-}
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
 
 template <int D, int QBLK, int MODE, bool HAS_V, bool STATS>
 __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {

@@ -17,17 +17,20 @@ namespace spattn {
 //   max_{r in W} (s[r,c] * sf - (max_q[r] * sf + log2 denom[r])) > log2 thresh.
 // Pad rows carry denom = -inf (include/maxq_denom.cuh:202-205) and never vote.
 //
-// One workgroup per q-block, each wave walks its own 32-key blocks.  Scores are S = Q K^T
-// with the query rows as the A operand - held in registers for d = 64 (each wave keeps
-// all 128 rows), read from an LDS copy of the tile for d = 128 - and the keys as the B
-// operand, loaded HBM -> registers one block ahead with no staging and no barrier.  The
-// accumulator of lane (n, g) holds key n against 64 of the 128 query rows.  The test is
-// rewritten once more as  s[r,c] - t[r] > 0  with the per-row constant
-// t[r] = (log2 thresh + max_q[r] sf + log2 denom[r]) / sf, and -t[r] is what the
-// accumulators start from: the matrix unit does the subtraction, the vector ALU only takes
-// the maximum of the 8 registers a lane holds of a 16-row group (v_max3) and compares it
-// with 0; one exchange with lane n^32 finishes the 8 votes of a key.  The vote count is
-// stored, not accumulated.
+// One workgroup per q-block, each wave walks its own 32-key blocks; no barrier in the
+// sweep.  Scores are S = Q K^T with the query rows as the A operand - held in registers for
+// d = 64 (each wave keeps all 128 rows), read from an LDS copy of the tile for d = 128 -
+// and the keys as the B operand.  For d = 64 every wave owns an LDS ring of four key
+// blocks that HBM -> LDS copies fill three blocks ahead (whole 128-byte rows per copy, the
+// swizzle applied by choosing which chunk a lane fetches); for d = 128, where the query
+// tile takes the LDS, the keys go HBM -> registers one block ahead.  The accumulator of
+// lane (n, g) holds key n against 64 of the 128 query rows.  The test is rewritten once
+// more as  s[r,c] - t[r] > 0  with the per-row constant
+// t[r] = (log2 thresh + max_q[r] sf + log2 denom[r]) / sf, and -t[r], kept in 64 registers,
+// is the C operand of the first multiply of every chain: the matrix unit does the
+// subtraction, the vector ALU only takes the maximum of the 8 registers a lane holds of a
+// 16-row group (v_max3) and compares it with 0; one exchange with lane n^32 finishes the 8
+// votes of a key.  The vote count is stored, not accumulated.
 // ------------------------------------------------------------------------------------
 template <int D>
 __global__ __launch_bounds__(256, 2) void booleanmask_kernel(int* __restrict__ mask, const float* __restrict__ max_q,
@@ -41,6 +44,11 @@ __global__ __launch_bounds__(256, 2) void booleanmask_kernel(int* __restrict__ m
   constexpr bool Q_REGS = (D == 64);
   __shared__ __attribute__((aligned(16))) unsigned char qs[Q_REGS ? 16 : 128 * D * 2];
   __shared__ __attribute__((aligned(16))) float nthr_l[2][4][16];   // [g][mb][register]
+  // d = 64: every wave owns a ring of four 4 KB key blocks, filled by HBM -> LDS copies
+  constexpr bool K_RING = Q_REGS;
+  constexpr int NSLOT = 4;
+  constexpr int KBLK = 32 * D * 2;
+  __shared__ __attribute__((aligned(1024))) unsigned char kring[K_RING ? 4 * NSLOT * KBLK : 16];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -79,8 +87,8 @@ __global__ __launch_bounds__(256, 2) void booleanmask_kernel(int* __restrict__ m
     }
   }
 
-  // Minus the per-row thresholds on the raw score, as a table in LDS from which the
-  // accumulators are initialised; register 4j+i of block mb in lane half g is query row
+  // Minus the per-row thresholds on the raw score, gathered through a table in LDS into the
+  // registers that start every multiply chain; register 4j+i of block mb in lane half g is query row
   // 32mb + 8j + 4g + i.  Pad rows and rows without keys get -inf and never vote.
   const float inv_sf = 1.f / sf;
   if (tid < 128) {
@@ -98,6 +106,46 @@ __global__ __launch_bounds__(256, 2) void booleanmask_kernel(int* __restrict__ m
 
   int* mrow = mask + ((size_t)bh * SB + qb) * mask_stride;
   const int nkb = (mask_stride + 31) >> 5;
+
+  // Ring layout: key row r of a block at r * 2D bytes, its 16-byte chunk c at c ^ kswz(r),
+  // which spreads chunk 2t+g of the 32 rows a half wave reads over all bank groups.  Copy i
+  // of a block moves rows 8i .. 8i+7: lane l fills position l of that 1 KB, i.e. fetches the
+  // chunk that belongs there, so that every copy reads eight whole rows of HBM.
+  auto kswz = [](int r) -> int { return (((r >> 1) & 1) << 2) | ((r >> 2) & 3); };
+  lds_cptr kread[K_RING ? NT : 1];     // per-lane read addresses inside slot 0 of this wave
+  int krow[K_RING ? 4 : 1];            // per-lane row of copy i inside a block
+  uint32_t kcol[K_RING ? 4 : 1];       // byte offset inside that row
+  const lds_cptr ring_l = (lds_cptr)kring + __builtin_amdgcn_readfirstlane(wave) * (NSLOT * KBLK);
+  const uint32_t ring_base = (uint32_t)(uintptr_t)ring_l;
+  if constexpr (K_RING) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) kread[t] = ring_l + ln * (D * 2) + (((2 * t + g) ^ kswz(ln)) << 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      krow[i] = 8 * i + (lane >> 3);
+      kcol[i] = ((lane & 7) ^ kswz(krow[i])) << 4;
+    }
+  }
+  // Rows past the end re-read the last key, blocks past the end likewise: every block costs
+  // the same four copies, which keeps the hand-counted waits valid up to the last block.
+  auto issue_keys = [&](int kb, int slot) {
+    if constexpr (K_RING) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        int key = kb * 32 + krow[i];
+        key = key < kv_len ? key : kv_len - 1;
+        dma16(kh, (uint32_t)key * (D * 2) + kcol[i],
+              __builtin_amdgcn_readfirstlane(ring_base + slot * KBLK + i * 1024));
+      }
+    }
+  };
+  auto slot_addr = [&](int slot) -> uint32_t { return (uint32_t)(slot & (NSLOT - 1)) * KBLK; };
+  auto read_keys = [&](int slot, u32x4 (&kf)[NT]) {
+    if constexpr (K_RING) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t) kf[t] = *(SPATTN_LDS const u32x4*)(kread[t] + slot_addr(slot));
+    }
+  };
 
   // Keys past the end re-read the last key (their votes are never stored): the loads are
   // unconditional, so the compiler can count them and let a block that was requested one
@@ -128,19 +176,21 @@ __global__ __launch_bounds__(256, 2) void booleanmask_kernel(int* __restrict__ m
   // while the matrix unit multiplies one pair, the vector ALU takes the maxima of the pair
   // before it, a few vector instructions behind every multiply, so that a wave is an even
   // mix of both at every point (two waves that alternate between a multiply-only and a
-  // vector-only phase fall into step and leave both units idle in turn).  Three accumulator
-  // sets rotate: multiplied now, reduced now, being initialised from the threshold table.
-  constexpr int NACC = Q_REGS ? 3 : 2;   // d = 128: registers for two sets only, the initialisation is then exposed
-  constexpr int NKS = Q_REGS ? 3 : 2;    // register sets of keys
+  // vector-only phase fall into step and leave both units idle in turn).
+  // Two accumulator sets alternate: multiplied now, reduced now.  The first multiply of a
+  // chain takes the threshold registers as its C operand and writes the set, so nothing has
+  // to be initialised.
+  constexpr int NACC = 2;
   f32x16 acc[NACC][2];
+  f32x16 nthr[4];
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb) nthr[mb] = *reinterpret_cast<const f32x16*>(&nthr_l[g][mb][0]);
   unsigned vhold = 0;
-  auto init_acc = [&](int p2, f32x16 (&dst)[2]) {
+  // reload: once a key register set has fed its last multiply of this block it is
+  // refilled from the ring slot of the wave's next block.
+  auto pair_scores = [&](int p2, u32x4 (&kf)[NT], f32x16 (&a2)[2], bool reload, uint32_t next_lds) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) dst[j] = *reinterpret_cast<const f32x16*>(&nthr_l[g][2 * p2 + j][0]);
-  };
-  auto pair_scores = [&](int p2, const u32x4 (&kf)[NT], f32x16 (&a2)[2]) {
-#pragma unroll
-    for (int t = 0; t < NT; ++t)
+    for (int t = 0; t < NT; ++t) {
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         const int mb = 2 * p2 + j;
@@ -148,8 +198,12 @@ __global__ __launch_bounds__(256, 2) void booleanmask_kernel(int* __restrict__ m
         u32x4 a;
         if constexpr (Q_REGS) a = qa[mb][t];
         else a = *reinterpret_cast<const u32x4*>(qs + qr * (D * 2) + (((2 * t + g) ^ swz(qr)) << 4));
-        a2[j] = mfma32(a, kf[t], a2[j]);
+        a2[j] = mfma32(a, kf[t], t == 0 ? nthr[mb] : a2[j]);
       }
+      if constexpr (K_RING) {
+        if (reload) kf[t] = *(SPATTN_LDS const u32x4*)(kread[t] + next_lds);
+      }
+    }
   };
   auto finish_block = [&](int kb, unsigned votes) {
     // A 16-row group is split over lanes n and n^32: it votes if either half does.
@@ -159,15 +213,12 @@ __global__ __launch_bounds__(256, 2) void booleanmask_kernel(int* __restrict__ m
     const int key = kb * 32 + ln;   // negative for the block "before the first": nothing is stored
     if (g == 0 && (unsigned)key < (unsigned)mask_stride) mrow[key] = (key < kv_len) ? __popc(votes) : 0;
   };
-  // Half H: multiplies pair H&1 of block kb into acc[H % NACC], reduces the accumulators of
-  // the half before, initialises those of the half after.
-  auto half = [&](auto hc, int kb, const u32x4 (&kf)[NT]) {
+  // Half H: multiplies pair H&1 of block kb into acc[H % NACC] and reduces the accumulators
+  // of the half before.
+  auto half = [&](auto hc, int kb, u32x4 (&kf)[NT], bool reload, uint32_t next_lds) {
     constexpr int H = decltype(hc)::value;
-    constexpr int P = H & 1, A = H % NACC, AP = (H + NACC - 1) % NACC, AN = (H + 1) % NACC;
-    // with three sets the one for the next half is free now: its initial values travel from
-    // LDS while this half is multiplied
-    if constexpr (NACC == 3) init_acc(1 - P, acc[AN]);
-    pair_scores(P, kf, acc[A]);
+    constexpr int P = H & 1, A = H % NACC, AP = (H + NACC - 1) % NACC;
+    pair_scores(P, kf, acc[A], reload, next_lds);
     const unsigned v = group_votes(2 * (1 - P), acc[AP][0]) | group_votes(2 * (1 - P) + 1, acc[AP][1]);
 #pragma unroll
     for (int i = 0; i < 2 * NT; ++i) {
@@ -175,7 +226,6 @@ __global__ __launch_bounds__(256, 2) void booleanmask_kernel(int* __restrict__ m
       __builtin_amdgcn_sched_group_barrier(0x002, (NT == 4) ? 3 : 2, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (NACC != 3) init_acc(1 - P, acc[AN]);
     if constexpr (P == 0) finish_block(kb - 4, vhold | v);   // pair 1 of the block before
     else vhold = v;                                          // pair 0 of this block
   };
@@ -186,61 +236,47 @@ __global__ __launch_bounds__(256, 2) void booleanmask_kernel(int* __restrict__ m
   };
   using I0 = std::integral_constant<int, 0>;
   using I1 = std::integral_constant<int, 1>;
-  using I2 = std::integral_constant<int, 2>;
-  using I3 = std::integral_constant<int, 3>;
-  using I4 = std::integral_constant<int, 4>;
-  using I5 = std::integral_constant<int, 5>;
 
-  // Key sets rotate without copies; a set is requested NKS-1 whole blocks before it is
-  // multiplied (a block is 4 NT multiplies, far shorter than a trip to L2).  The main loop
-  // runs whole rotations without side exits; at most NKS-1 blocks remain after it.
   int kb = wave;
-  init_acc(0, acc[0]);
-  init_acc(1, acc[NACC - 1]);   // reduced by the very first half; its votes go nowhere
-  if constexpr (NKS == 3) {
-    u32x4 k0[NT], k1[NT], k2[NT];
-    load_keys(kb, k0);
-    load_keys(kb + 4, k1);
-    while (kb + 8 < nkb) {
-      load_keys(kb + 8, k2);
-      half(I0{}, kb, k0);
-      half(I1{}, kb, k0);
-      load_keys(kb + 12, k0);
-      half(I2{}, kb + 4, k1);
-      half(I3{}, kb + 4, k1);
-      load_keys(kb + 16, k1);
-      half(I4{}, kb + 8, k2);
-      half(I5{}, kb + 8, k2);
-      kb += 12;
-    }
-    if (kb < nkb) {
-      half(I0{}, kb, k0);
-      half(I1{}, kb, k0);
-      if (kb + 4 < nkb) {
-        half(I2{}, kb + 4, k1);
-        half(I3{}, kb + 4, k1);
-        drain(std::integral_constant<int, 3 % NACC>{}, kb + 4);
-      } else {
-        drain(std::integral_constant<int, 1 % NACC>{}, kb);
-      }
-    } else {
-      drain(std::integral_constant<int, 5 % NACC>{}, kb - 4);
-    }
+  acc[1][0] = nthr[2];   // reduced by the very first half; its votes go nowhere
+  acc[1][1] = nthr[3];
+  if constexpr (K_RING) {
+    // The copies of a block go out three of the wave's blocks ahead; the registers of block
+    // b+1 are read from the ring during the second half of block b.  Of the vector-memory
+    // operations that follow the copies of block b+1 in program order, the 8 copies of the
+    // blocks b+2 and b+3 are always there (vote stores may or may not be), hence vmcnt(8).
+    u32x4 kf[NT];
+    int slot = 0;
+    issue_keys(kb, 0);
+    issue_keys(kb + 4, 1);
+    issue_keys(kb + 8, 2);
+    wait_vmcnt<8>();
+    read_keys(0, kf);
+    auto block = [&](auto h0, auto h1, int kbb) {
+      issue_keys(kbb + 12, (slot + 3) & (NSLOT - 1));
+      half(h0, kbb, kf, false, 0u);
+      wait_vmcnt<8>();
+      half(h1, kbb, kf, true, slot_addr(slot + 1));
+      slot = (slot + 1) & (NSLOT - 1);
+    };
+    for (; kb < nkb; kb += 4) block(I0{}, I1{}, kb);
+    drain(I1{}, kb - 4);
+    wait_vmcnt<0>();   // no copy may land after the workgroup has given up its LDS
   } else {
     u32x4 k0[NT], k1[NT];
     load_keys(kb, k0);
     while (kb + 4 < nkb) {
       load_keys(kb + 4, k1);
-      half(I0{}, kb, k0);
-      half(I1{}, kb, k0);
+      half(I0{}, kb, k0, false, 0u);
+      half(I1{}, kb, k0, false, 0u);
       load_keys(kb + 8, k0);
-      half(I0{}, kb + 4, k1);
-      half(I1{}, kb + 4, k1);
+      half(I0{}, kb + 4, k1, false, 0u);
+      half(I1{}, kb + 4, k1, false, 0u);
       kb += 8;
     }
     if (kb < nkb) {
-      half(I0{}, kb, k0);
-      half(I1{}, kb, k0);
+      half(I0{}, kb, k0, false, 0u);
+      half(I1{}, kb, k0, false, 0u);
       drain(I1{}, kb);
     } else {
       drain(I1{}, kb - 4);
