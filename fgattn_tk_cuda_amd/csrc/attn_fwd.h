@@ -50,16 +50,14 @@ typedef __attribute__((ext_vector_type(4))) short s16x4;
 template <int D, int MODE, bool HAS_V>
 struct AttnCfg {
   static constexpr int kTileBytes = 64 * D * 2;
-  // Ring slots: K tiles are copied three tiles ahead (two with token lists, whose key
-  // validity ring shares the 80 KB that let two workgroups share a CU), V tiles one ahead.
-  static constexpr int kKSlots = (MODE == KV_TOKENS) ? 2 : 3;
+  // Ring slots: K tiles are copied three tiles ahead, V tiles one ahead; 80 KB at d = 128,
+  // which lets two workgroups share a CU.
+  static constexpr int kKSlots = 3;
   static constexpr int kVSlots = HAS_V ? 2 : 0;
   static constexpr int kSlots = kKSlots + kVSlots;
-  static constexpr int kBiasRing = 8;                         // tiles of key-validity bias (token lists)
-  static constexpr int kBiasBytes = (MODE == KV_TOKENS) ? kBiasRing * 64 * 4 : 0;
   static constexpr int kRing = kSlots * kTileBytes;
   static constexpr int kMerge = 2 * (D / 2 + 3) * 64 * 4;     // key-split merge, overlays the ring
-  static constexpr int kTotal = ((kRing > kMerge) ? kRing : kMerge) + kBiasBytes;
+  static constexpr int kTotal = (kRing > kMerge) ? kRing : kMerge;
   static constexpr int kRowsPerLoad = 1024 / (D * 2);         // rows one wave-wide 1 KB load covers
   static constexpr int kLoadsPerTile = kTileBytes / 1024 / 4;   // per wave
 };
@@ -171,72 +169,57 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     return start | (keys << 24);
   };
 
-  // Token lists: the RPL token ids behind one load are wave-uniform, so they are fetched
-  // as scalars (tok_raw) one tile ahead and turned into this lane's row (tok_row) just
-  // before the K load of that tile is issued; V tiles are issued one tile later and take
-  // their rows from a two-deep queue.
-  int tok_raw[MODE == KV_TOKENS ? LPT : 1][MODE == KV_TOKENS ? RPL : 1];
-  int tok_row[MODE == KV_TOKENS ? LPT : 1];      // rows of the next K tile to issue
-  int tok_row_v0[MODE == KV_TOKENS ? LPT : 1];   // rows of the next V tile to issue
-  int tok_row_v1[MODE == KV_TOKENS ? LPT : 1];   // rows of the V tile after that
-  bool tok_ok[MODE == KV_TOKENS ? LPT : 1];
-  auto tok_fetch = [&](int t) {
+  // Token lists: lane l of every wave fetches entry 64t + l of the list, one tile further
+  // ahead than the K copies (ids_load: a vector load written as asm, so that it is counted
+  // by hand like the tile copies).  When the K copy of tile t is prepared, the entries that
+  // name a key (position < n, id < kv_len) are balloted into the tile's 64-bit key mask,
+  // the others are pointed at row 0, and each copy takes the row of its lane from the
+  // lane that holds it (ds_bpermute).  idr / idw / idh hold ids and mask halves of tile j
+  // at index j % 6.
+  int idr[MODE == KV_TOKENS ? 6 : 1] = {};
+  uint64_t lst_addr = 0;
+  if constexpr (MODE == KV_TOKENS) {
+    const uint64_t a = (uint64_t)(uintptr_t)(p.idx + ((size_t)bh * p.nqblk + qb) * p.idx_stride);
+    // readfirstlane returns a signed int: without the casts the low word would be sign-extended
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)a);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+    lst_addr = ((uint64_t)hi << 32) | lo;
+  }
+  auto ids_load = [&](int t, int& dst) {
     if constexpr (MODE == KV_TOKENS) {
-#pragma unroll
-      for (int i = 0; i < LPT; ++i)
-#pragma unroll
-        for (int s = 0; s < RPL; ++s) tok_raw[i][s] = (t < ntiles) ? lst[t * 64 + RPL * (4 * i + wave) + s] : 0;
+      int pos = t * 64 + lane;
+      pos = pos < p.idx_stride ? pos : p.idx_stride - 1;
+      asm volatile("global_load_dword %0, %1, %2" : "=v"(dst) : "v"(pos * 4), "s"(lst_addr) : "memory");
     }
   };
-  auto tok_resolve = [&](int t) {
+  auto ids_resolve = [&](int t, int& ids, int& mlo, int& mhi) {
     if constexpr (MODE == KV_TOKENS) {
-#pragma unroll
-      for (int i = 0; i < LPT; ++i) {
-        int tok = 0;
-#pragma unroll
-        for (int s = 0; s < RPL; ++s) {
-          int v = tok_raw[i][s];
-          v = __builtin_amdgcn_readfirstlane(v);   // keeps the list a scalar load (no per-lane reload)
-          tok = (ld_sub == s) ? v : tok;
-        }
-        tok_ok[i] = (t * 64 + ld_row(i)) < n && (unsigned)tok <= (unsigned)last_row;
-        tok_row[i] = tok_ok[i] ? tok : 0;
-      }
+      const bool ok = (t * 64 + lane) < n && (unsigned)ids <= (unsigned)last_row;
+      const unsigned long long m = __ballot(ok);
+      mlo = (int)(unsigned)m;
+      mhi = (int)(unsigned)(m >> 32);
+      ids = ok ? ids : 0;
     }
   };
 
   // Loads of one K or V tile into ring slot `slot`: prepare() resolves the wave-uniform
   // base and this lane's byte offsets, load(i) issues the i-th of the LPT wave-wide copies.
-  // With token lists the tiles are issued K0 K1 V0 K2 V1 ..., which the token-row queue relies on.
   struct TileLoad {
     const unsigned char* base;
     uint32_t lds;
     uint32_t go[LPT];
   };
-  auto prepare_tile = [&](int t, int desc, int slot, bool is_v) -> TileLoad {
+  // desc: tile descriptor (dense / block lists) or the resolved ids of the tile (token lists)
+  auto prepare_tile = [&](int desc, int slot, bool is_v) -> TileLoad {
     TileLoad tl;
     tl.lds = smem_base + (uint32_t)slot * TILE + wave * 1024;
     const unsigned char* src = is_v ? vh : kh;
     if constexpr (MODE == KV_TOKENS) {
       tl.base = src;
-      float* bias = reinterpret_cast<float*>(smem + Cfg::kTotal - Cfg::kBiasBytes) + (t % Cfg::kBiasRing) * 64;
 #pragma unroll
       for (int i = 0; i < LPT; ++i) {
-        const int row = is_v ? tok_row_v0[i] : tok_row[i];
+        const int row = __builtin_amdgcn_ds_bpermute(ld_row(i) * 4, desc);
         tl.go[i] = (uint32_t)row * ROWB + ld_off(i);
-        if (!is_v && ld_slot == 0) bias[ld_row(i)] = tok_ok[i] ? 0.f : kNegInf;
-      }
-      if (is_v) {
-#pragma unroll
-        for (int i = 0; i < LPT; ++i) tok_row_v0[i] = tok_row_v1[i];
-      } else {
-#pragma unroll
-        for (int i = 0; i < LPT; ++i) {
-          if (t == 0) tok_row_v0[i] = tok_row[i];
-          tok_row_v1[i] = tok_row[i];
-        }
-        tok_resolve(t + 1);
-        tok_fetch(t + 2);
       }
     } else {
       tl.base = src + (size_t)(desc & 0xffffff) * ROWB;
@@ -246,8 +229,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     return tl;
   };
   auto load_part = [&](const TileLoad& tl, int i) { dma16(tl.base, tl.go[i], tl.lds + i * 4096); };
-  auto issue_tile = [&](int t, int slot, bool is_v) {
-    const TileLoad tl = prepare_tile(t, tile_desc(t), slot, is_v);
+  auto issue_tile = [&](int desc, int slot, bool is_v) {
+    const TileLoad tl = prepare_tile(desc, slot, is_v);
 #pragma unroll
     for (int i = 0; i < LPT; ++i) load_part(tl, i);
   };
@@ -260,12 +243,24 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   auto kslot = [](int t) -> int { return t % NK; };
   auto vslot = [](int t) -> int { return NK + (t & 1); };
 
-  // Copies go out in the order K0 K1 V0 K2 | V1 K3 | V2 K4 | ... (three K slots) or
-  // K0 K1 V0 | K2 V1 | K3 V2 | ... (two K slots, token lists).
-  tok_fetch(0);
-  tok_resolve(0);
-  tok_fetch(1);
-  if (ntiles > 0) issue_tile(0, kslot(0), false);
+  // Copies go out in the order K0 K1 V0 K2 | V1 K3 | V2 K4 | ...
+  int idw[6] = {0, 0, 0, 0, 0, 0};   // descriptors (key mask, low half) of the tiles in flight, tile j in idw[j % 6]
+  int idh[6] = {0, 0, 0, 0, 0, 0};   // token lists: key mask, high half
+  if constexpr (MODE == KV_TOKENS) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) ids_load(j, idr[j]);
+    wait_vmcnt<0>();
+#pragma unroll
+    for (int j = 0; j < 4; ++j) asm volatile("" : "+v"(idr[j]));
+#pragma unroll
+    for (int j = 0; j < 3; ++j) ids_resolve(j, idr[j], idw[j], idh[j]);
+  }
+  // what prepare_tile takes for tile j (a prologue tile: j < 3)
+  auto head_desc = [&](int j) -> int {
+    if constexpr (MODE == KV_TOKENS) return idr[j];
+    else return tile_desc(j);
+  };
+  if (ntiles > 0) issue_tile(head_desc(0), kslot(0), false);
   // The Q loads are the only compiler-visible vector loads of the kernel.  They go out
   // between the first copies so that their latency overlaps that of tile 0, and must have
   // retired before the first counted wait.
@@ -277,9 +272,9 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   }
   int head_pending = 0;   // tile copies behind K0 when the first phase waits
   if (ntiles > 0) {
-    if (1 < ntiles) { issue_tile(1, kslot(1), false); ++head_pending; }
-    if constexpr (HAS_V) { issue_tile(0, vslot(0), true); ++head_pending; }
-    if (NK == 3 && 2 < ntiles) { issue_tile(2, kslot(2), false); ++head_pending; }
+    if (1 < ntiles) { issue_tile(head_desc(1), kslot(1), false); ++head_pending; }
+    if constexpr (HAS_V) { issue_tile(head_desc(0), vslot(0), true); ++head_pending; }
+    if (NK == 3 && 2 < ntiles) { issue_tile(head_desc(2), kslot(2), false); ++head_pending; }
   }
 #pragma unroll
   for (int t = 0; t < NT; ++t) asm volatile("" ::"v"(qf[t]));
@@ -345,19 +340,19 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   // ---- building blocks --------------------------------------------------------------
   // Keys of tile `it` that do not exist get -inf.  Accumulator register 4j+i of block mb
   // is key ksub*KW + 32mb + 8j + 4g + i of the tile.
-  auto mask_tile = [&](int it, int desc, f32x16 (&s)[NMB]) {
+  auto mask_tile = [&](int desc, int desc_hi, f32x16 (&s)[NMB]) {
     if constexpr (MODE == KV_TOKENS) {
-      const float* bias = reinterpret_cast<const float*>(smem + Cfg::kTotal - Cfg::kBiasBytes) + (it % Cfg::kBiasRing) * 64;
+      if ((desc & desc_hi) != -1) {   // wave-uniform: some key of the tile does not exist
+        const unsigned long long m = ((unsigned long long)(unsigned)desc_hi << 32) | (unsigned)desc;
+        const unsigned long long mine = m >> (ksub * KW + 4 * g);   // bit c: this lane's key c
 #pragma unroll
-      for (int mb = 0; mb < NMB; ++mb)
+        for (int mb = 0; mb < NMB; ++mb)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float4 bv = *reinterpret_cast<const float4*>(bias + ksub * KW + 32 * mb + 8 * j + 4 * g);
-          s[mb][4 * j + 0] += bv.x;
-          s[mb][4 * j + 1] += bv.y;
-          s[mb][4 * j + 2] += bv.z;
-          s[mb][4 * j + 3] += bv.w;
-        }
+          for (int r = 0; r < 16; ++r) {
+            const int c = 32 * mb + 8 * (r >> 2) + (r & 3);
+            if (!((mine >> c) & 1)) s[mb][r] = kNegInf;
+          }
+      }
     } else {
       const int keys = desc >> 24;
       if (keys < 64) {
@@ -564,7 +559,6 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   };
 
   f32x16 s_e[NMB], s_o[NMB];   // scores of even / odd tiles
-  int idw[6] = {0, 0, 0, 0, 0, 0};   // descriptors of tiles it+1 .. it+NK(+1), tile j in idw[j % 6]
 
   // One tile of the pipeline, between two barriers: the scores of tile it+1 are multiplied
   // (K slot (it+1) % NK) while the softmax of tile it runs on the vector ALU, then P V of
@@ -581,21 +575,32 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     const bool has_kn = it + NK < ntiles;
     // behind K(it+1) and V(it) only K(it+2) can be in flight (three K slots)
     if (NK == 3 && it + 2 < ntiles) wait_vmcnt<LPT>(); else wait_vmcnt<0>();
+    if constexpr (MODE == KV_TOKENS) {
+      // the ids of tile it+NK, requested one tile ago, are behind the wait above
+      asm volatile("" : "+v"(idr[(KC + NK) % 6]));
+      ids_resolve(it + NK, idr[(KC + NK) % 6], idw[(KC + NK) % 6], idh[(KC + NK) % 6]);
+    }
     __syncthreads();
     v_addr_refresh();
-    const int d_v = idw[(KC + 1) % 6];
-    const int d_k = idw[(KC + NK) % 6];
-    constexpr bool K_FIRST = (MODE == KV_TOKENS) || !HAS_V;   // token rows are queued K first
-    const TileLoad tl_first = K_FIRST ? prepare_tile(it + NK, d_k, KN, false) : prepare_tile(it + 1, d_v, VN, true);
+    // what the copies of V(it+1) and K(it+NK) are prepared from, and the key mask of tile it+1
+    const int d_v = (MODE == KV_TOKENS) ? idr[(KC + 1) % 6] : idw[(KC + 1) % 6];
+    const int d_k = (MODE == KV_TOKENS) ? idr[(KC + NK) % 6] : idw[(KC + NK) % 6];
+    const int m_lo = idw[(KC + 1) % 6], m_hi = idh[(KC + 1) % 6];
+    constexpr bool K_FIRST = !HAS_V;
+    const TileLoad tl_first = K_FIRST ? prepare_tile(d_k, KN, false) : prepare_tile(d_v, VN, true);
     qk_tile(std::true_type{}, std::integral_constant<bool, HAS_V>{}, KS * TILE, VS * TILE, s_b, s_a, &tl_first,
             K_FIRST ? has_kn : true);
+    // ids of tile it+NK+1: between the copies of V(it+1) and K(it+NK) in the order of issue.
+    // Issued whether or not that tile exists (the position is clamped to the list): the wait
+    // counts stay the same on every tile, and the registers are held until the final wait.
+    if constexpr (MODE == KV_TOKENS) ids_load(it + NK + 1, idr[(KC + NK + 1) % 6]);
     softmax_close(s_a);
-    mask_tile(it + 1, d_v, s_b);
+    mask_tile(m_lo, m_hi, s_b);
     if constexpr (MODE != KV_TOKENS) idw[(KC + NK + 1) % 6] = tile_desc(it + NK + 1);
     float mloc_sf;
     using stat_t = std::integral_constant<bool, !LAZY_MAX>;
     if constexpr (HAS_V) {
-      const TileLoad tl_second = K_FIRST ? prepare_tile(it + 1, d_v, VN, true) : prepare_tile(it + NK, d_k, KN, false);
+      const TileLoad tl_second = K_FIRST ? prepare_tile(d_v, VN, true) : prepare_tile(d_k, KN, false);
       mloc_sf = pv_tile(std::true_type{}, stat_t{}, VS * TILE, &tl_second, K_FIRST ? true : has_kn, s_b);
     } else {
       mloc_sf = pv_tile(std::true_type{}, stat_t{}, 0, nullptr, false, s_b);
@@ -617,7 +622,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     else wait_vmcnt<0>();
     __syncthreads();
     qk_tile(std::false_type{}, std::false_type{}, 0, 0, s_e, s_e, nullptr, false);
-    mask_tile(0, tile_desc(0), s_e);
+    if constexpr (MODE == KV_TOKENS) mask_tile(idw[0], idh[0], s_e);
+    else mask_tile(tile_desc(0), 0, s_e);
     maybe_rescale(row_stats(s_e));
 
     int it = 0;
@@ -651,8 +657,13 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     }
     // tail: softmax and P V of the last tile
     if (it & 1) { softmax_only(s_o); softmax_close(s_o); } else { softmax_only(s_e); softmax_close(s_e); }
+    wait_vmcnt<0>();
+    if constexpr (MODE == KV_TOKENS) {
+      // the id registers stay allocated until every id load has landed
+#pragma unroll
+      for (int j = 0; j < 6; ++j) asm volatile("" ::"v"(idr[j]));
+    }
     if constexpr (HAS_V) {
-      wait_vmcnt<0>();
       __syncthreads();
       v_addr_refresh();
       pv_tile(std::false_type{}, std::false_type{}, (uint32_t)(it & 1) * TILE, nullptr, false, s_e);
