@@ -65,6 +65,33 @@ def test_sp_attn_ragged_token_lists(dev, D, qblk):
     assert_close_stat(lse, wl_, "lse vs oracle")
 
 
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("qblk", [64, 128])
+def test_sp_attn_long_lists_with_entries_that_name_no_key(dev, D, qblk):
+    """Lists of 13 to 25 tiles in which one entry in twelve is negative or past the end:
+    such entries are skipped wherever they stand, also in the steady part of the tile loop."""
+    print("case sp_attn holes", D, qblk, flush=True)
+    B, H, S = 1, 3, 1600
+    rng = np.random.default_rng(15)
+    q, k, v = wl.randn_qkv(B, H, S, D, seed=16)
+    ms = orc.padded_len(S)
+    nq = orc.ceil_div(S, qblk)
+    idx = np.full((B, H, nq, ms), ms, np.int32)
+    num = np.zeros((B, H, nq), np.int32)
+    for h in range(H):
+        for i in range(nq):
+            c = int(rng.integers(800, S))
+            lst = rng.permutation(S)[:c].astype(np.int32)
+            holes = rng.random(c) < 1.0 / 12
+            lst[holes] = rng.choice(np.array([-1, -7, S, S + 5, 2 ** 30], np.int32), int(holes.sum()))
+            idx[0, h, i, :c] = lst
+            num[0, h, i] = c
+    o, lse = _run_tokens(dev, q, k, v, torch.from_numpy(idx), torch.from_numpy(num), qblk)
+    wo, wl_ = orc.sp_attn(f32(q), f32(k), f32(v), idx, num, qblk=qblk)
+    assert_close_o(o, wo, "O vs oracle")
+    assert_close_stat(lse, wl_, "lse vs oracle")
+
+
 def test_sp_attn_single_key_returns_v_row(dev):
     print("case sp_attn single key", flush=True)
     B, H, S, D = 1, 1, 256, 128
