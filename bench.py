@@ -95,6 +95,17 @@ def bench_sparse(dev, steps, warmup, seed=0):
                 count=count, tensors=(q, k, v, bi, bc, o))
 
 
+def bench_tokens(dev, steps, warmup, seed=0, res=None):
+    """The headline workload handed over the way the reference operator takes it: the same
+    kept keys as token-id lists kv_indices [B,H,S/64,S] int32 + counts (sp_attn)."""
+    res = res or bench_sparse(dev, 2, 1, seed=seed)
+    q, k, v, bi, bc, o = res["tensors"]
+    S, qblk = res["S"], res["qblk"]
+    tok, num = (t.to(dev) for t in wl.blocks_to_tokens(bi.cpu(), bc.cpu(), S))
+    ms, _ = time_steps(lambda: capi.sp_attn(o, q, k, v, tok, num, qblk=qblk), steps, warmup)
+    return dict(ms=ms, flops=res["flops"], list_bytes=4.0 * tok.numel())
+
+
 def bench_compaction(dev, steps, warmup, seed=0):
     """booleanmask_to_indexmask at the padded threshold workload: B=1, H=24, N=32760 -> mask
     [1,24,256,32768] int32 with ~8 % of the entries set."""
@@ -217,7 +228,7 @@ def main(argv=None) -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-extras", action="store_true", help="only the headline kernel")
-    ap.add_argument("--only", default="", help="run one leg only: sparse|compact|dense|sweeps|copy|packed (no JSON contract)")
+    ap.add_argument("--only", default="", help="run one leg only: sparse|tokens|compact|dense|sweeps|copy|packed (no JSON contract)")
     args = ap.parse_args(argv)
     if args.gpus != 1:
         print("bench.py: this library is single-GPU; run with --gpus 1 (got %d)" % args.gpus, file=sys.stderr)
@@ -231,7 +242,7 @@ def main(argv=None) -> int:
 
     if args.only:
         fn = {"sparse": bench_sparse, "compact": bench_compaction, "dense": bench_dense, "sweeps": bench_sweeps,
-              "copy": bench_copy, "packed": bench_packed}[args.only]
+              "copy": bench_copy, "packed": bench_packed, "tokens": bench_tokens}[args.only]
         r = fn(dev, args.steps, args.warmup)
         r.pop("tensors", None)
         print(json.dumps(r))
@@ -253,6 +264,11 @@ def main(argv=None) -> int:
                      "kernel": "attn_fwd_kernel<128,64,KV_BLOCKS>"},
     }
     if not args.no_extras:
+        tk = bench_tokens(dev, args.steps, args.warmup, res=res)
+        out["token_lists"] = {"workload": "cfg3 with the kept keys as token-id lists (the reference operator's form)",
+                              "kernel": "attn_fwd_kernel<128,64,KV_TOKENS>", "ms": tk["ms"],
+                              "tflops": tk["flops"] / (tk["ms"] * 1e-3) / 1e12,
+                              "mfma_frac": tk["flops"] / (tk["ms"] * 1e-3) / 1e12 / PEAK_BF16_TFLOPS}
         cp = bench_compaction(dev, args.steps, args.warmup)
         gbps = cp["bytes"] / (cp["ms"] * 1e-3) / 1e9
         out["mask_pass"] = {"kernel": "compact_kernel (booleanmask_to_indexmask)", "workload": "cfg4 mask %s int32, %.1f%% kept"
