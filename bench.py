@@ -149,6 +149,28 @@ def bench_packed(dev, steps, warmup, seed=0):
                 ms_index=ms_idx, bytes_index=rows * ms_ / 8.0 + 4.0 * kept + 4.0 * rows, kept=kept)
 
 
+def bench_topk(dev, steps, warmup, seed=0):
+    """The top-k mask generator at the threshold workload's shape (B=1, H=24, N=32760, d=64,
+    128-row q-blocks), keeping 8 % of the keys per q-block: q-block means, one product per
+    head, a radix select per row.  Bytes: q and k once, the bf16 score matrix written and read
+    once, the lists written."""
+    c = wl.CONFIGS["cfg4_threshold_padded"]
+    B, H, S, D = c["B"], c["H"], c["S"], c["D"]
+    q, k, _ = (t.to(dev) for t in wl.clustered_qkv(B, H, S, D, seed=seed))
+    SB = wl.ceil_div(S, 128)
+    Sp = 128 * SB
+    select_k = int(round(c["keep"] * S))
+    stride = 128 * wl.ceil_div(select_k, 128)
+    kvi = torch.full((B, H, SB, stride), stride, dtype=torch.int32, device=dev)
+    kvn = torch.zeros((B, H, SB), dtype=torch.int32, device=dev)
+    score = torch.empty((B, H, SB, Sp), dtype=torch.bfloat16, device=dev)
+    qmean = torch.empty((B, H, SB, D), dtype=torch.bfloat16, device=dev)
+    ms, _ = time_steps(lambda: capi.qk_topkmask_indices(kvi, kvn, score, qmean, q, k, select_k, blocksz=128), steps, warmup)
+    rows = B * H * SB
+    nbytes = 2.0 * (q.numel() + k.numel()) + 2.0 * qmean.numel() + 2 * 2.0 * rows * S + 4.0 * rows * select_k + 4.0 * rows
+    return dict(ms=ms, bytes=nbytes, select_k=select_k, rows=rows)
+
+
 def bench_copy(dev, steps, warmup, seed=0):
     """A plain 1 GiB device-to-device copy: the known-size kernel that the FETCH_SIZE /
     WRITE_SIZE counters of the other kernels are scaled by."""
@@ -228,7 +250,7 @@ def main(argv=None) -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-extras", action="store_true", help="only the headline kernel")
-    ap.add_argument("--only", default="", help="run one leg only: sparse|tokens|compact|dense|sweeps|copy|packed (no JSON contract)")
+    ap.add_argument("--only", default="", help="run one leg only: sparse|tokens|compact|dense|sweeps|copy|packed|topk (no JSON contract)")
     args = ap.parse_args(argv)
     if args.gpus != 1:
         print("bench.py: this library is single-GPU; run with --gpus 1 (got %d)" % args.gpus, file=sys.stderr)
@@ -242,7 +264,7 @@ def main(argv=None) -> int:
 
     if args.only:
         fn = {"sparse": bench_sparse, "compact": bench_compaction, "dense": bench_dense, "sweeps": bench_sweeps,
-              "copy": bench_copy, "packed": bench_packed, "tokens": bench_tokens}[args.only]
+              "copy": bench_copy, "packed": bench_packed, "tokens": bench_tokens, "topk": bench_topk}[args.only]
         r = fn(dev, args.steps, args.warmup)
         r.pop("tensors", None)
         print(json.dumps(r))
@@ -284,6 +306,10 @@ def main(argv=None) -> int:
             "packedmask_to_indexmask_ms": pk["ms_index"], "packedmask_to_indexmask_gbps": pk["bytes_index"] / pk["ms_index"] / 1e6,
             "packedmask_to_indexmask_hbm_frac": pk["bytes_index"] / pk["ms_index"] / 1e6 / PEAK_HBM_GBPS,
             "algorithmic_bytes": [pk["bytes_pack"], pk["bytes_index"]]}
+        tp = bench_topk(dev, max(2, args.steps // 4), 2)
+        out["topk_mask"] = {"workload": "cfg4 shape, q-block-mean top-k, %d keys per q-block" % tp["select_k"],
+                            "ms": tp["ms"], "gbps": tp["bytes"] / tp["ms"] / 1e6,
+                            "hbm_frac": tp["bytes"] / tp["ms"] / 1e6 / PEAK_HBM_GBPS, "algorithmic_bytes": tp["bytes"]}
         dn = bench_dense(dev, args.steps, args.warmup)
         out["dense_full_attn"] = {"workload": "cfg2: B=4 H=16 N=4096 d=64", "ms": dn["ms"],
                                   "tflops": dn["flops"] / (dn["ms"] * 1e-3) / 1e12,

@@ -37,6 +37,7 @@ _SIGNATURES = {
     "spattn_booleanmask_to_indexmask": (_c_int, [_c_void_p] * 3 + [_c_int] * 5 + [_c_void_p]),
     "spattn_pack_mask": (_c_int, [_c_void_p] * 2 + [_c_int] * 4 + [_c_void_p]),
     "spattn_packedmask_to_indexmask": (_c_int, [_c_void_p] * 3 + [_c_int] * 5 + [_c_void_p]),
+    "spattn_qk_topkmask_indices": (_c_int, [_c_void_p] * 6 + [_c_int] * 9 + [_c_void_p]),
     "spattn_last_status": (_c_int, []),
     "spattn_status_string": (ctypes.c_char_p, [_c_int]),
     "spattn_version": (_c_int, []),
@@ -198,6 +199,25 @@ def packedmask_to_indexmask(kv_indices, kv_num_indices, packed, seq, *, stream=N
         raise ValueError("kv_indices / kv_num_indices do not match the packed mask")
     _check(load().spattn_packedmask_to_indexmask(_ptr(kv_indices, i32), _ptr(kv_num_indices, i32),
                                                  _ptr(packed, torch.uint8), B, H, int(seq), SB, MS, _stream(stream)))
+
+
+def qk_topkmask_indices(kv_indices, kv_num_indices, score, qmean, q, k, select_k, *, blocksz=128, kv_len=0,
+                        stream=None):
+    """Top-k keys per q-block by (block-mean query / sqrt(D)) . key; ascending key lists.
+    score: bf16 [B,H,SB,score_stride] and qmean: bf16 [B,H,SB,D] are outputs as well."""
+    B, H, S, D = (int(x) for x in q.shape)
+    SB = (S + blocksz - 1) // blocksz
+    if tuple(k.shape) != (B, H, S, D):
+        raise ValueError("k must match q")
+    if tuple(qmean.shape) != (B, H, SB, D) or score.dim() != 4 or tuple(score.shape[:3]) != (B, H, SB):
+        raise ValueError("qmean must be [B,H,SB,D] and score [B,H,SB,score_stride]")
+    if kv_indices.dim() != 4 or tuple(kv_indices.shape[:3]) != (B, H, SB) or kv_num_indices.numel() != B * H * SB:
+        raise ValueError("kv_indices must be [B,H,SB,idx_stride] and kv_num_indices hold B*H*SB entries")
+    bf = torch.bfloat16
+    _check(load().spattn_qk_topkmask_indices(_ptr(kv_indices, i32), _ptr(kv_num_indices, i32), _ptr(score, bf),
+                                             _ptr(qmean, bf), _ptr(q, bf), _ptr(k, bf), B, H, S, D, int(blocksz),
+                                             int(kv_len), int(select_k), int(score.shape[3]),
+                                             int(kv_indices.shape[3]), _stream(stream)))
 
 
 def infer_qblk(seq: int, seqblocks: int) -> int:

@@ -162,6 +162,24 @@ int spattn_packedmask_to_indexmask(int* kv_indices, int* num_kv_indices, const v
                                                   B * H * seqblocks, mask_stride, seq, as_stream(stream)));
 }
 
+int spattn_qk_topkmask_indices(int* kv_indices, int* num_kv_indices, void* score, void* qmean, const void* q,
+                               const void* k, int batch, int heads, int seq, int D, int blocksz, int kv_len,
+                               int select_k, int score_stride, int idx_stride, void* stream) {
+  if (!kv_indices || !num_kv_indices || !score || !qmean || !q || !k) return done(SPATTN_ERR_NULL);
+  if (D != 64 && D != 128) return done(SPATTN_ERR_HEAD_DIM);
+  if (batch <= 0 || heads <= 0 || seq <= 0 || select_k <= 0) return done(SPATTN_ERR_SHAPE);
+  if (blocksz != 64 && blocksz != 128) return done(SPATTN_ERR_QBLK);
+  if (kv_len < 0 || kv_len > seq) return done(SPATTN_ERR_SHAPE);
+  const int kv = kv_len > 0 ? kv_len : seq;
+  if (score_stride < kv || score_stride % 8 != 0) return done(SPATTN_ERR_STRIDE);
+  if (idx_stride < (select_k < kv ? select_k : kv)) return done(SPATTN_ERR_STRIDE);
+  if (misaligned(score) || misaligned(qmean) || misaligned(q) || misaligned(k)) return done(SPATTN_ERR_ALIGN);
+  return from_hip(spattn::run_topk_mask(kv_indices, num_kv_indices, static_cast<uint16_t*>(score),
+                                        static_cast<uint16_t*>(qmean), static_cast<const uint16_t*>(q),
+                                        static_cast<const uint16_t*>(k), batch, heads, seq, D, blocksz, kv, select_k,
+                                        score_stride, idx_stride, as_stream(stream)));
+}
+
 // ---- the reference's binding surface: default stream, default scale, q-block 128 ----
 
 void attn_fwd_wg_impl(void* o, void* q, void* k, void* v, int batch, int heads, int seq, int D) {

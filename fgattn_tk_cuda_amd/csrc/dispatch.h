@@ -22,4 +22,9 @@ hipError_t run_pack_mask(uint32_t* packed, const int* mask, int rows, int mask_s
 hipError_t run_packed_to_indexmask(int* kv_indices, int* kv_num, const uint32_t* packed, int rows, int mask_stride,
                                    int kv_len, hipStream_t stream);
 
+// topk_kernels.hip
+hipError_t run_topk_mask(int* kv_indices, int* kv_num, uint16_t* score, uint16_t* qmean, const uint16_t* q,
+                         const uint16_t* k, int B, int H, int S, int D, int blk, int kv_len, int select_k,
+                         int score_stride, int idx_stride, hipStream_t stream);
+
 }  // namespace spattn

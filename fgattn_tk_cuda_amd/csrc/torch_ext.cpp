@@ -195,6 +195,37 @@ void packedmask_to_indexmask(torch::Tensor kv_indices, torch::Tensor kv_numindic
                "packedmask_to_indexmask");
 }
 
+// The top-k mask generator of the reference's Python layer (python/spattn/mask_utils.py:389-417)
+// as one operator: q-block means, their scores against every key, and the select_k best keys
+// per q-block as ascending lists.  score and qmean are outputs too.
+void qk_topkmask_indices(torch::Tensor kv_indices, torch::Tensor kv_numindices, torch::Tensor score, torch::Tensor qmean,
+                         torch::Tensor q, torch::Tensor k, int64_t select_k, int64_t blocksz) {
+  TORCH_CHECK(q.is_cuda() && q.scalar_type() == at::kBFloat16 && q.is_contiguous() && q.dim() == 4,
+              "q must be a contiguous bf16 device tensor [B,H,S,D]");
+  check_aux(k, "k", at::kBFloat16, q);
+  check_aux(score, "score", at::kBFloat16, q);
+  check_aux(qmean, "qmean", at::kBFloat16, q);
+  check_aux(kv_indices, "kv_indices", at::kInt, q);
+  check_aux(kv_numindices, "kv_numindices", at::kInt, q);
+  TORCH_CHECK(k.sizes() == q.sizes(), "k must match q");
+  TORCH_CHECK(blocksz > 0, "blocksz must be positive");
+  const int64_t B = q.size(0), H = q.size(1), S = q.size(2), D = q.size(3);
+  const int64_t SB = (S + blocksz - 1) / blocksz;
+  TORCH_CHECK(qmean.dim() == 4 && qmean.size(0) == B && qmean.size(1) == H && qmean.size(2) == SB && qmean.size(3) == D,
+              "qmean must be [B,H,SB,D]");
+  TORCH_CHECK(score.dim() == 4 && score.size(0) == B && score.size(1) == H && score.size(2) == SB,
+              "score must be [B,H,SB,score_stride]");
+  TORCH_CHECK(kv_indices.dim() == 4 && kv_indices.size(0) == B && kv_indices.size(1) == H && kv_indices.size(2) == SB,
+              "kv_indices must be [B,H,SB,idx_stride]");
+  TORCH_CHECK(kv_numindices.numel() == B * H * SB, "kv_numindices must have B*H*SB entries");
+  const DeviceGuard guard(q.device());
+  check_status(spattn_qk_topkmask_indices(kv_indices.data_ptr<int>(), kv_numindices.data_ptr<int>(), score.data_ptr(),
+                                          qmean.data_ptr(), q.data_ptr(), k.data_ptr(), (int)B, (int)H, (int)S, (int)D,
+                                          (int)blocksz, 0, (int)select_k, (int)score.size(3), (int)kv_indices.size(3),
+                                          cur_stream()),
+               "qk_topkmask_indices");
+}
+
 // Meta kernels: shapes only, nothing to compute (all ops mutate their arguments in place).
 void noop4(torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor) {}
 void noop_all_index(torch::Tensor, torch::Tensor, int64_t, int64_t, int64_t, int64_t) {}
@@ -202,6 +233,7 @@ void noop6(torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Te
 void noop_mask(torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, double) {}
 void noop_b2i(torch::Tensor, torch::Tensor, torch::Tensor, int64_t) {}
 void noop2(torch::Tensor, torch::Tensor) {}
+void noop_topk(torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, int64_t, int64_t) {}
 
 TORCH_LIBRARY_FRAGMENT(cuda_attn, m) {
   m.def("full_attn(Tensor(a!) o, Tensor q, Tensor k, Tensor v) -> ()");
@@ -213,6 +245,7 @@ TORCH_LIBRARY_FRAGMENT(cuda_attn, m) {
   m.def("booleanmask_to_indexmask(Tensor(a!) kv_indices, Tensor(b!) kv_numindices, Tensor booleanmask, int seq) -> ()");
   m.def("pack_mask(Tensor(a!) packed, Tensor booleanmask) -> ()");
   m.def("packedmask_to_indexmask(Tensor(a!) kv_indices, Tensor(b!) kv_numindices, Tensor packed, int seq) -> ()");
+  m.def("qk_topkmask_indices(Tensor(a!) kv_indices, Tensor(b!) kv_numindices, Tensor(c!) score, Tensor(d!) qmean, Tensor q, Tensor k, int select_k, int blocksz) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(cuda_attn, Meta, m) {
@@ -225,6 +258,7 @@ TORCH_LIBRARY_IMPL(cuda_attn, Meta, m) {
   m.impl("booleanmask_to_indexmask", noop_b2i);
   m.impl("pack_mask", noop2);
   m.impl("packedmask_to_indexmask", noop_b2i);
+  m.impl("qk_topkmask_indices", noop_topk);
 }
 
 // The CUDA dispatch key serves HIP tensors on PyTorch-ROCm.
@@ -238,6 +272,7 @@ TORCH_LIBRARY_IMPL(cuda_attn, CUDA, m) {
   m.impl("booleanmask_to_indexmask", booleanmask_to_indexmask);
   m.impl("pack_mask", pack_mask);
   m.impl("packedmask_to_indexmask", packedmask_to_indexmask);
+  m.impl("qk_topkmask_indices", qk_topkmask_indices);
 }
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -250,4 +285,5 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("fullattn_maxq_denom", &fullattn_maxq_denom, "fullattn_maxq_denom");
   m.def("pack_mask", &pack_mask, "pack_mask");
   m.def("packedmask_to_indexmask", &packedmask_to_indexmask, "packedmask_to_indexmask");
+  m.def("qk_topkmask_indices", &qk_topkmask_indices, "qk_topkmask_indices");
 }

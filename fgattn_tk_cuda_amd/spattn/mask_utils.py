@@ -273,6 +273,26 @@ def qk_topkmask_indices(q, k, select_k, blocksz=128):
     return kv_indices, torch.full((B, H, nb), select_k, device=q.device, dtype=torch.int32)
 
 
+def qk_topkmask_indices_cuda(q, k, select_k, blocksz=128):
+    """The same selection on the device in three kernels (q-block means, one [SB x D].[D x S]
+    product per head, a radix select per row): kv_indices [B,H,SB,stride] int32 with the
+    select_k keys of each q-block in ascending order, stride = select_k rounded up to 128 and
+    the tail filled with stride, and kv_num_indices.  Every step is rounded to bf16 as the
+    reference's bf16 torch ops are (python/spattn/mask_utils.py:390-413); among equal scores
+    the lower key wins."""
+    B, H, S, D = q.shape
+    nb = (S + blocksz - 1) // blocksz
+    select_k = min(int(select_k), S)
+    stride = _padded(select_k)
+    kv_indices = torch.full((B, H, nb, stride), stride, dtype=torch.int32, device=q.device)
+    kv_num_indices = torch.empty((B, H, nb), dtype=torch.int32, device=q.device)
+    score = torch.empty((B, H, nb, _padded(S)), dtype=torch.bfloat16, device=q.device)
+    qmean = torch.empty((B, H, nb, D), dtype=torch.bfloat16, device=q.device)
+    spattn_interface.qk_topkmask_indices(kv_indices, kv_num_indices, score, qmean, q.contiguous(), k.contiguous(),
+                                         select_k, blocksz)
+    return kv_indices, kv_num_indices
+
+
 # ----------------------------------------------------------------------------------
 # bit packing (python/spattn/mask_utils.py:421-439)
 # ----------------------------------------------------------------------------------

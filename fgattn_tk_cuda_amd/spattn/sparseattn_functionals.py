@@ -55,14 +55,10 @@ def attn_computed_with_sparse_mask_python(query, key, value, current_layer=None,
 
 
 def attn_topkmask_cuda(query, key, value, current_layer=None, ditrun=None, *args, **kwargs):
-    """Top-k key lists per q-block, then sparse attention (:39-48).  The sparse operator
-    needs lists padded to a multiple of 128 keys."""
+    """Top-k key lists per q-block, then sparse attention (:39-48).  The lists come from the
+    device selector, padded to a multiple of 128 keys as the sparse operator needs."""
     select_k = kwargs.get("select_k") or query.shape[2]
-    kv_indices, kv_num_indices = mask_utils.qk_topkmask_indices(query, key, select_k, blocksz=kwargs["blocksz"])
-    stride = mask_utils._padded(select_k)
-    if stride != select_k:
-        pad = torch.full((*kv_indices.shape[:3], stride - select_k), stride, dtype=torch.int32, device=query.device)
-        kv_indices = torch.cat([kv_indices, pad], dim=-1)
+    kv_indices, kv_num_indices = mask_utils.qk_topkmask_indices_cuda(query, key, select_k, blocksz=kwargs["blocksz"])
     return _sparse(query, key, value, kv_indices, kv_num_indices)
 
 

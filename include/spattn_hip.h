@@ -121,6 +121,19 @@ int spattn_pack_mask(void* packed, const int* booleanmask, int batch, int heads,
 int spattn_packedmask_to_indexmask(int* kv_indices, int* num_kv_indices, const void* packed, int batch, int heads,
                                    int seq, int seqblocks, int mask_stride, void* stream);
 
+/* Top-k mask generator (python/spattn/mask_utils.py:389-417, qk_topkmask_indices): per
+ * q-block of `blocksz` rows the select_k keys c < kv_len (0 = seq) with the largest
+ * (block mean of q / sqrt(D)) . k[c], every step rounded to bf16 as the reference's bf16 torch
+ * ops do.  Outputs: qmean bf16 [batch,heads,SB,D]; score bf16 [batch,heads,SB,score_stride]
+ * (columns >= kv_len are not written; score_stride a multiple of 8); kv_indices
+ * [batch,heads,SB,idx_stride] receives min(select_k, kv_len) keys per row in ASCENDING key
+ * order (the reference orders them by descending score; sp_attn does not depend on the
+ * order), entries behind them keep the caller's fill; num_kv_indices the count.  Among equal
+ * scores the lower key wins.  SB = ceil(seq / blocksz), blocksz 64 or 128. */
+int spattn_qk_topkmask_indices(int* kv_indices, int* num_kv_indices, void* score, void* qmean, const void* q,
+                               const void* k, int batch, int heads, int seq, int D, int blocksz, int kv_len,
+                               int select_k, int score_stride, int idx_stride, void* stream);
+
 /* Status of the most recent call on this host thread, and its text. */
 int spattn_last_status(void);
 const char* spattn_status_string(int status);

@@ -21,6 +21,11 @@ pinned (none of them is "parity unpinned"):
 * ``booleanmask_to_indexmask`` - integer exact; ``np.flatnonzero`` per row and
   a pure-Python loop on small inputs.
 * ``all_index_mask``           - ``arange`` closed form (include/utils.cuh:73-93).
+* ``pack_mask`` / ``unpack_mask`` / ``packedmask_to_indexmask`` - ``numpy.packbits`` and round trips.
+* ``qblock_mean_scores``       - the reference's own torch expressions
+  (python/spattn/mask_utils.py:390-410) evaluated in bf16 on the CPU.
+* ``topk_select``              - the multiset of selected scores equals
+  ``torch.topk(...).values`` (python/spattn/mask_utils.py:412); brute force on tiny rows.
 """
 from __future__ import annotations
 
@@ -296,3 +301,42 @@ def packedmask_to_indexmask(packed, seq, fill=None):
     """unpack followed by booleanmask_to_indexmask: what CompressedBitMaskCache.get_mask_from_cache
     computes (python/spattn/mask_utils.py:86-90)."""
     return booleanmask_to_indexmask(unpack_mask(packed).astype(np.int32), seq, fill=fill)
+
+
+def qblock_mean_scores(q, k, blocksz: int = 128):
+    """qmean and score of the top-k mask generator, with the roundings of the reference's bf16
+    torch ops (python/spattn/mask_utils.py:390-410): block mean (fp32 sum * 1/rows -> bf16),
+    divided by sqrt(D) (-> bf16), fp32 dot with every key (-> bf16).
+    q, k: [B,H,S,D] holding bf16-representable values.  Returns (qmean [B,H,SB,D], score [B,H,SB,S])."""
+    q = np.asarray(q, np.float32)
+    k = np.asarray(k, np.float32)
+    B, H, S, D = q.shape
+    SB = ceil_div(S, blocksz)
+    qmean = np.zeros((B, H, SB, D), np.float32)
+    for m in range(SB):
+        blk = q[:, :, m * blocksz:(m + 1) * blocksz]
+        rows = blk.shape[2]
+        acc = np.zeros((B, H, D), np.float32)
+        for r in range(rows):              # row after row in fp32, the order of the device kernel
+            acc = acc + blk[:, :, r]
+        qmean[:, :, m] = bf16_round(acc * (np.float32(1.0) / np.float32(rows)))
+    qmean = bf16_round(qmean / np.float32(math.sqrt(D)))
+    score = bf16_round(np.einsum("bhmd,bhnd->bhmn", qmean, k).astype(np.float32))
+    return qmean, score
+
+
+def topk_select(score, select_k: int, kv_len: int | None = None):
+    """The select_k keys c < kv_len with the largest score per row, larger score first and the
+    lower key first among equal scores (torch.topk, python/spattn/mask_utils.py:412, leaves
+    the order among equal scores open), returned as ASCENDING key lists.
+    score: [..., S].  Returns int32 [..., min(select_k, kv_len)]."""
+    score = np.asarray(score, np.float32)
+    S = score.shape[-1]
+    kv_len = S if kv_len is None else kv_len
+    kk = min(select_k, kv_len)
+    flat = score.reshape(-1, S)[:, :kv_len]
+    out = np.zeros((flat.shape[0], kk), np.int32)
+    for i, row in enumerate(flat):
+        order = np.lexsort((np.arange(kv_len), -row))   # by score descending, then key ascending
+        out[i] = np.sort(order[:kk])
+    return out.reshape(*score.shape[:-1], kk)

@@ -225,3 +225,50 @@ def test_pack_mask_matches_library_and_round_trips():
     wi, wn = orc.packedmask_to_indexmask(packed, 200)
     ri, rn = orc.booleanmask_to_indexmask(mask, 200)
     assert np.array_equal(wi, ri) and np.array_equal(wn, rn)
+
+
+@pytest.mark.parametrize("S,D,blk", [(300, 64, 128), (256, 128, 64), (130, 128, 128)])
+def test_topk_generator_scores_match_the_reference_expressions_in_bf16(S, D, blk):
+    """qmean / score of the oracle against the reference's own torch expressions
+    (python/spattn/mask_utils.py:390-410) evaluated in bf16 on the CPU: qmean exact, score
+    equal except where another summation order moves a value across a bf16 rounding boundary."""
+    g = torch.Generator().manual_seed(S + D)
+    B, H = 1, 2
+    q = torch.randn(B, H, S, D, generator=g).bfloat16()
+    k = torch.randn(B, H, S, D, generator=g).bfloat16()
+    qm, sc = orc.qblock_mean_scores(q.float().numpy(), k.float().numpy(), blk)
+    fl = S // blk
+    full = q[:, :, :fl * blk].view(B, H, fl, blk, D).mean(dim=3)
+    parts = [full]
+    if S % blk:
+        parts.append(q[:, :, fl * blk:].mean(dim=2, keepdim=True))
+    qs = torch.cat(parts, dim=2) * 1. / D ** 0.5
+    ut = torch.einsum("bhmd,bhnd->bhmn", qs, k)
+    assert np.array_equal(qm, qs.float().numpy())
+    want = ut.float().numpy()
+    diff = sc != want
+    assert diff.mean() < 0.01
+    assert np.all(np.abs(sc - want)[diff] <= np.abs(want[diff]) * 2.0 ** -7 + 1e-30)
+
+
+def test_topk_select_matches_torch_topk_values_and_brute_force():
+    rng = np.random.default_rng(4)
+    # bf16-like scores with many ties
+    sc = orc.bf16_round(rng.standard_normal((3, 5, 700)).astype(np.float32))
+    for kk in (1, 37, 128, 700, 900):
+        sel = orc.topk_select(sc, kk)
+        k_eff = min(kk, 700)
+        assert sel.shape == (3, 5, k_eff) and np.all(np.diff(sel, axis=-1) > 0)
+        mine = np.take_along_axis(sc, sel.astype(np.int64), -1)
+        want = torch.topk(torch.from_numpy(sc), k_eff, dim=-1).values.numpy()
+        assert np.array_equal(np.sort(mine, -1), np.sort(want, -1))
+    # ties go to the lower key; kv_len cuts the candidates
+    row = np.array([[1.0, 3.0, 3.0, 2.0, 3.0, 3.0, 0.5, 9.0]], np.float32)
+    assert orc.topk_select(row, 3).tolist() == [[1, 2, 7]]
+    assert orc.topk_select(row, 3, kv_len=6).tolist() == [[1, 2, 4]]
+    # brute force on tiny rows
+    for _ in range(50):
+        r = orc.bf16_round(rng.integers(-3, 4, size=(1, 12)).astype(np.float32))
+        kk = int(rng.integers(1, 13))
+        pairs = sorted(((-float(r[0, i]), i) for i in range(12)))[:kk]
+        assert orc.topk_select(r, kk)[0].tolist() == sorted(i for _, i in pairs)
