@@ -149,7 +149,7 @@ def bench_packed(dev, steps, warmup, seed=0):
                 ms_index=ms_idx, bytes_index=rows * ms_ / 8.0 + 4.0 * kept + 4.0 * rows, kept=kept)
 
 
-def bench_topk(dev, steps, warmup, seed=0):
+def bench_topk(dev, steps, warmup, seed=0, score_pad=0):
     """The top-k mask generator at the threshold workload's shape (B=1, H=24, N=32760, d=64,
     128-row q-blocks), keeping 8 % of the keys per q-block: q-block means, one product per
     head, a radix select per row.  Bytes: q and k once, the bf16 score matrix written and read
@@ -163,7 +163,7 @@ def bench_topk(dev, steps, warmup, seed=0):
     stride = 128 * wl.ceil_div(select_k, 128)
     kvi = torch.full((B, H, SB, stride), stride, dtype=torch.int32, device=dev)
     kvn = torch.zeros((B, H, SB), dtype=torch.int32, device=dev)
-    score = torch.empty((B, H, SB, Sp), dtype=torch.bfloat16, device=dev)
+    score = torch.empty((B, H, SB, Sp + score_pad), dtype=torch.bfloat16, device=dev)
     qmean = torch.empty((B, H, SB, D), dtype=torch.bfloat16, device=dev)
     ms, _ = time_steps(lambda: capi.qk_topkmask_indices(kvi, kvn, score, qmean, q, k, select_k, blocksz=128), steps, warmup)
     rows = B * H * SB

@@ -125,7 +125,7 @@ int spattn_packedmask_to_indexmask(int* kv_indices, int* num_kv_indices, const v
  * q-block of `blocksz` rows the select_k keys c < kv_len (0 = seq) with the largest
  * (block mean of q / sqrt(D)) . k[c], every step rounded to bf16 as the reference's bf16 torch
  * ops do.  Outputs: qmean bf16 [batch,heads,SB,D]; score bf16 [batch,heads,SB,score_stride]
- * (columns >= kv_len are not written; score_stride a multiple of 8); kv_indices
+ * (columns >= kv_len hold unspecified values; score_stride a multiple of 8); kv_indices
  * [batch,heads,SB,idx_stride] receives min(select_k, kv_len) keys per row in ASCENDING key
  * order (the reference orders them by descending score; sp_attn does not depend on the
  * order), entries behind them keep the caller's fill; num_kv_indices the count.  Among equal

@@ -316,9 +316,15 @@ def qblock_mean_scores(q, k, blocksz: int = 128):
     for m in range(SB):
         blk = q[:, :, m * blocksz:(m + 1) * blocksz]
         rows = blk.shape[2]
-        acc = np.zeros((B, H, D), np.float32)
-        for r in range(rows):              # row after row in fp32, the order of the device kernel
-            acc = acc + blk[:, :, r]
+        # fp32 order of the device kernel: 512 / D interleaved row phases, each summed row
+        # after row, then the phases added in order
+        phases = 512 // D
+        acc = None
+        for j in range(phases):
+            part = np.zeros((B, H, D), np.float32)
+            for r in range(j, rows, phases):
+                part = part + blk[:, :, r]
+            acc = part if acc is None else acc + part
         qmean[:, :, m] = bf16_round(acc * (np.float32(1.0) / np.float32(rows)))
     qmean = bf16_round(qmean / np.float32(math.sqrt(D)))
     score = bf16_round(np.einsum("bhmd,bhnd->bhmn", qmean, k).astype(np.float32))

@@ -53,6 +53,20 @@ def test_topk_generator_matches_oracle(dev, D, blk, S, select_k, kv_len):
     assert np.all(kvi[..., kk:] == fill)
 
 
+def test_topk_rows_longer_than_the_lds_path(dev):
+    """More than 72000 keys per row: the select that re-reads its row from memory."""
+    print("case topk long rows", flush=True)
+    B, H, S, D, blk, select_k = 1, 1, 81000, 64, 128, 700
+    q, k, _ = wl.randn_qkv(B, H, S, D, seed=5)
+    kvi, kvn, score, qmean, fill = _run(dev, q, k, select_k, blk)
+    want_qm, _ = orc.qblock_mean_scores(f32(q)[:, :, :256], f32(k)[:, :, :256], blk)
+    assert np.array_equal(qmean[:, :, :2], want_qm[:, :, :2])
+    rows = [0, 1, 317, 632]
+    want_sel = orc.topk_select(score[0, 0, rows, :S], select_k)
+    assert np.all(kvn == select_k)
+    assert np.array_equal(kvi[0, 0, rows, :select_k], want_sel)
+
+
 def test_topk_select_ties_and_wide_rows(dev):
     """Constant keys give equal scores everywhere: the lowest keys win; a second head with
     two score levels checks the boundary between the levels."""
