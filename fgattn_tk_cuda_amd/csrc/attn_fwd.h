@@ -761,12 +761,9 @@ template <int D, int QBLK, int MODE, bool HAS_V, bool STATS>
 inline hipError_t launch_attn_fwd(const AttnParams& p, hipStream_t stream) {
   using Cfg = AttnCfg<D, MODE, HAS_V>;
   auto kern = attn_fwd_kernel<D, QBLK, MODE, HAS_V, STATS>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kTotal);
-    if (e != hipSuccess) return e;
-    attr_set = true;
-  }
+  static bool attr_set[kMaxDevices] = {};
+  const hipError_t ea = raise_lds_limit(reinterpret_cast<const void*>(kern), Cfg::kTotal, attr_set);
+  if (ea != hipSuccess) return ea;
   const int total = p.nqblk * p.H * p.B;
   if (total <= 0) return hipSuccess;
   hipLaunchKernelGGL(kern, dim3(total), dim3(256), Cfg::kTotal, stream, p);

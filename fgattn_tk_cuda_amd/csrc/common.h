@@ -110,4 +110,18 @@ __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
+// Raises a kernel's dynamic-LDS limit once per device (the attribute belongs to the device's
+// copy of the kernel).  Host only; racing threads repeat a call that does no harm.
+constexpr int kMaxDevices = 64;
+inline hipError_t raise_lds_limit(const void* kernel, int bytes, bool (&done)[kMaxDevices]) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev >= 0 && dev < kMaxDevices && done[dev]) return hipSuccess;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) return e;
+  if (dev >= 0 && dev < kMaxDevices) done[dev] = true;
+  return hipSuccess;
+}
+
 }  // namespace spattn

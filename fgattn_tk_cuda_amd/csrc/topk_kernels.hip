@@ -549,13 +549,10 @@ hipError_t run_topk_mask(int* kv_indices, int* kv_num, uint16_t* score, uint16_t
   }
   if (kv_len <= kTopkLdsMaxKeys) {
     const int lds = 16 * ((kv_len + 7) / 8) + kTopkLdsExtra;
-    static int attr_lds = 0;   // largest size the attribute has been raised to (same value from every thread)
-    if (lds > attr_lds) {
-      e = hipFuncSetAttribute(reinterpret_cast<const void*>(topk_select_lds_kernel),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, 16 * (kTopkLdsMaxKeys / 8) + kTopkLdsExtra);
-      if (e != hipSuccess) return e;
-      attr_lds = 16 * (kTopkLdsMaxKeys / 8) + kTopkLdsExtra;
-    }
+    static bool attr_set[kMaxDevices] = {};
+    e = raise_lds_limit(reinterpret_cast<const void*>(topk_select_lds_kernel),
+                        16 * (kTopkLdsMaxKeys / 8) + kTopkLdsExtra, attr_set);
+    if (e != hipSuccess) return e;
     const int grid = rows < 8192 ? rows : 8192;
     hipLaunchKernelGGL(topk_select_lds_kernel, dim3(grid), dim3(kTopkThreads), lds, stream, kv_indices, kv_num, score, rows,
                        score_stride, kv_len, select_k, idx_stride);
