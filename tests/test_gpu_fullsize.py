@@ -26,6 +26,37 @@ def _oracle_block_rows(q, k, v, bi, bc, b, h, i, qblk, S):
     return (p @ f32(v[b, h])[lst]) / den[:, None], m * np.float32(scale) + np.log(den)
 
 
+def test_cfg1_plumbing_case_against_dense_masked_softmax(dev):
+    """B=1 H=4 N=1024 d=64, fp32 Q/K/V ~ N(0,1), 64x64 blocks, diagonal + random key blocks up
+    to 25 % per q-block row: O = softmax(QK^T / 8 masked to -inf outside the kept blocks) V,
+    computed densely in fp32 on the host, against the device kernel (block lists and token
+    lists) on the same values rounded to bf16."""
+    print("case cfg1 plumbing", flush=True)
+    from oracle import cpu_masked_attention as cma
+
+    c = wl.CONFIGS["cfg1_plumbing"]
+    B, H, S, D, qblk, kvblk = c["B"], c["H"], c["S"], c["D"], c["qblk"], c["kvblk"]
+    q32, k32, v32 = wl.randn_qkv(B, H, S, D, seed=101, dtype=torch.float32)
+    q, k, v = q32.bfloat16(), k32.bfloat16(), v32.bfloat16()
+    bi, bc = wl.uniform_block_lists(B, H, S, qblk, kvblk, int(round(c["density"] * (S // kvblk))), seed=102)
+    qd, kd, vd, bid, bcd = to_dev(dev, q, k, v, bi, bc)
+    o = torch.empty_like(qd)
+    lse = torch.empty((B, H, S), device=dev)
+    capi.sp_attn_blocks(o, qd, kd, vd, bid, bcd, lse=lse, qblk=qblk)
+    tok, num = wl.blocks_to_tokens(bi, bc, S)
+    o2 = torch.empty_like(qd)
+    capi.sp_attn(o2, qd, kd, vd, tok.to(dev), num.to(dev), qblk=qblk)
+    torch.cuda.synchronize()
+    for h in range(H):
+        want = cma.masked_attention_rows(q[0, h].float(), k[0, h].float(), v[0, h].float(), bi[0, h], bc[0, h], 0, S,
+                                         qblk, kvblk)
+        assert_close_o(f32(o[0, h]), f32(want), "cfg1 block lists, head %d" % h)
+        assert_close_o(f32(o2[0, h]), f32(want), "cfg1 token lists, head %d" % h)
+        # the bf16 rounding of the inputs is the only difference from the fp32 definition
+        want32 = cma.masked_attention_rows(q32[0, h], k32[0, h], v32[0, h], bi[0, h], bc[0, h], 0, S, qblk, kvblk)
+        assert np.abs(f32(o[0, h]) - f32(want32)).max() < 6e-2
+
+
 def test_cfg3_headline_shape(dev):
     """B=2 H=32 N=16384 d=128, 26 of 256 blocks per 64-row q-block."""
     print("case cfg3 full size", flush=True)

@@ -272,3 +272,22 @@ def test_topk_select_matches_torch_topk_values_and_brute_force():
         kk = int(rng.integers(1, 13))
         pairs = sorted(((-float(r[0, i]), i) for i in range(12)))[:kk]
         assert orc.topk_select(r, kk)[0].tolist() == sorted(i for _, i in pairs)
+
+
+def test_cfg1_plumbing_case_oracle_equals_dense_masked_softmax():
+    """The CPU-runnable configuration (B=1 H=4 N=1024 d=64 fp32, 64x64 blocks, diagonal plus
+    random key blocks up to 25 %): the oracle's gathered form equals the dense definition
+    softmax(QK^T * scale with -inf outside the kept blocks) V evaluated with torch in fp32."""
+    c = wl.CONFIGS["cfg1_plumbing"]
+    B, H, S, D, qblk, kvblk = c["B"], c["H"], c["S"], c["D"], c["qblk"], c["kvblk"]
+    q, k, v = wl.randn_qkv(B, H, S, D, seed=101, dtype=torch.float32)
+    bi, bc = wl.uniform_block_lists(B, H, S, qblk, kvblk, int(round(c["density"] * (S // kvblk))), seed=102)
+    assert bi.shape[-1] == 4 and all(i in bi[0, 0, i].tolist() for i in range(S // qblk))
+    tok, num = wl.blocks_to_tokens(bi, bc, S)
+    got, lse = orc.sp_attn(q.numpy(), k.numpy(), v.numpy(), tok.numpy(), num.numpy(), qblk=qblk, round_p=False)
+    for h in range(H):
+        want = cma.masked_attention_rows(q[0, h], k[0, h], v[0, h], bi[0, h], bc[0, h], 0, S, qblk, kvblk)
+        assert np.abs(got[0, h] - want.numpy()).max() < 2e-5
+        s = (q[0, h] @ k[0, h].T) * D ** -0.5
+        s.masked_fill_(~cma.block_mask_rows(bi[0, h], bc[0, h], 0, S, qblk, kvblk, S), float("-inf"))
+        assert np.abs(lse[0, h] - torch.logsumexp(s, -1).numpy()).max() < 2e-5
