@@ -209,8 +209,13 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     uint32_t lds;
     uint32_t go[LPT];
   };
-  // desc: tile descriptor (dense / block lists) or the resolved ids of the tile (token lists)
-  auto prepare_tile = [&](int desc, int slot, bool is_v) -> TileLoad {
+  // desc: tile descriptor (dense / block lists) or the resolved ids of the tile (token lists).
+  // Token lists with a 64-row q-block (registers to spare): the byte offsets found for the K
+  // copy of tile j are kept in gor[j % 3] and serve its V copy two tiles later.
+  constexpr bool GO_RING = (MODE == KV_TOKENS) && HAS_V && QBLK == 64;
+  uint32_t gor[GO_RING ? 3 : 1][GO_RING ? LPT : 1];
+  auto prepare_tile = [&](int desc, int slot, bool is_v, auto gic) -> TileLoad {
+    constexpr int GI = decltype(gic)::value;
     TileLoad tl;
     tl.lds = smem_base + (uint32_t)slot * TILE + wave * 1024;
     const unsigned char* src = is_v ? vh : kh;
@@ -218,8 +223,13 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
       tl.base = src;
 #pragma unroll
       for (int i = 0; i < LPT; ++i) {
-        const int row = __builtin_amdgcn_ds_bpermute(ld_row(i) * 4, desc);
-        tl.go[i] = (uint32_t)row * ROWB + ld_off(i);
+        if (GO_RING && is_v) {
+          tl.go[i] = gor[GO_RING ? GI : 0][GO_RING ? i : 0];
+        } else {
+          const int row = __builtin_amdgcn_ds_bpermute(ld_row(i) * 4, desc);
+          tl.go[i] = (uint32_t)row * ROWB + ld_off(i);
+          if constexpr (GO_RING) gor[GI][i] = tl.go[i];
+        }
       }
     } else {
       tl.base = src + (size_t)(desc & 0xffffff) * ROWB;
@@ -229,8 +239,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     return tl;
   };
   auto load_part = [&](const TileLoad& tl, int i) { dma16(tl.base, tl.go[i], tl.lds + i * 4096); };
-  auto issue_tile = [&](int desc, int slot, bool is_v) {
-    const TileLoad tl = prepare_tile(desc, slot, is_v);
+  auto issue_tile = [&](int desc, int slot, bool is_v, auto gic) {
+    const TileLoad tl = prepare_tile(desc, slot, is_v, gic);
 #pragma unroll
     for (int i = 0; i < LPT; ++i) load_part(tl, i);
   };
@@ -260,7 +270,10 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     if constexpr (MODE == KV_TOKENS) return idr[j];
     else return tile_desc(j);
   };
-  if (ntiles > 0) issue_tile(head_desc(0), kslot(0), false);
+  using G0 = std::integral_constant<int, 0>;
+  using G1 = std::integral_constant<int, 1>;
+  using G2 = std::integral_constant<int, 2>;
+  if (ntiles > 0) issue_tile(head_desc(0), kslot(0), false, G0{});
   // The Q loads are the only compiler-visible vector loads of the kernel.  They go out
   // between the first copies so that their latency overlaps that of tile 0, and must have
   // retired before the first counted wait.
@@ -272,9 +285,9 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   }
   int head_pending = 0;   // tile copies behind K0 when the first phase waits
   if (ntiles > 0) {
-    if (1 < ntiles) { issue_tile(head_desc(1), kslot(1), false); ++head_pending; }
-    if constexpr (HAS_V) { issue_tile(head_desc(0), vslot(0), true); ++head_pending; }
-    if (NK == 3 && 2 < ntiles) { issue_tile(head_desc(2), kslot(2), false); ++head_pending; }
+    if (1 < ntiles) { issue_tile(head_desc(1), kslot(1), false, G1{}); ++head_pending; }
+    if constexpr (HAS_V) { issue_tile(head_desc(0), vslot(0), true, G0{}); ++head_pending; }
+    if (NK == 3 && 2 < ntiles) { issue_tile(head_desc(2), kslot(2), false, G2{}); ++head_pending; }
   }
 #pragma unroll
   for (int t = 0; t < NT; ++t) asm volatile("" ::"v"(qf[t]));
@@ -587,7 +600,9 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     const int d_k = (MODE == KV_TOKENS) ? idr[(KC + NK) % 6] : idw[(KC + NK) % 6];
     const int m_lo = idw[(KC + 1) % 6], m_hi = idh[(KC + 1) % 6];
     constexpr bool K_FIRST = !HAS_V;
-    const TileLoad tl_first = K_FIRST ? prepare_tile(d_k, KN, false) : prepare_tile(d_v, VN, true);
+    using GK = std::integral_constant<int, (KC + NK) % 3>;    // tile it+NK
+    using GV = std::integral_constant<int, (KC + 1) % 3>;     // tile it+1
+    const TileLoad tl_first = K_FIRST ? prepare_tile(d_k, KN, false, GK{}) : prepare_tile(d_v, VN, true, GV{});
     qk_tile(std::true_type{}, std::integral_constant<bool, HAS_V>{}, KS * TILE, VS * TILE, s_b, s_a, &tl_first,
             K_FIRST ? has_kn : true);
     // ids of tile it+NK+1: between the copies of V(it+1) and K(it+NK) in the order of issue.
@@ -600,7 +615,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     float mloc_sf;
     using stat_t = std::integral_constant<bool, !LAZY_MAX>;
     if constexpr (HAS_V) {
-      const TileLoad tl_second = K_FIRST ? prepare_tile(d_v, VN, true) : prepare_tile(d_k, KN, false);
+      const TileLoad tl_second = K_FIRST ? prepare_tile(d_v, VN, true, GV{}) : prepare_tile(d_k, KN, false, GK{});
       mloc_sf = pv_tile(std::true_type{}, stat_t{}, VS * TILE, &tl_second, K_FIRST ? true : has_kn, s_b);
     } else {
       mloc_sf = pv_tile(std::true_type{}, stat_t{}, 0, nullptr, false, s_b);
