@@ -176,7 +176,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   // the others are pointed at row 0, and each copy takes the row of its lane from the
   // lane that holds it (ds_bpermute).  idr / idw / idh hold ids and mask halves of tile j
   // at index j % 6.
-  int idr[MODE == KV_TOKENS ? 6 : 1] = {};
+  int idr[6] = {};   // used with token lists only
   uint64_t lst_addr = 0;
   if constexpr (MODE == KV_TOKENS) {
     const uint64_t a = (uint64_t)(uintptr_t)(p.idx + ((size_t)bh * p.nqblk + qb) * p.idx_stride);
