@@ -106,6 +106,28 @@ def bench_tokens(dev, steps, warmup, seed=0, res=None):
     return dict(ms=ms, flops=res["flops"], list_bytes=4.0 * tok.numel())
 
 
+def bench_zipf(dev, steps, warmup, seed=0):
+    """cfg5: B=1 H=8 N=65536 d=128, 128-row q-blocks, per-row block counts ~ Zipf(1.2) clipped to
+    [1,1024]: the default schedule against the longest-list-first work order (same results)."""
+    c = wl.CONFIGS["cfg5_zipf_64k"]
+    B, H, S, D, qblk = c["B"], c["H"], c["S"], c["D"], c["qblk"]
+    q, k, v = (t.to(dev) for t in wl.randn_qkv(B, H, S, D, seed=seed))
+    cnt = wl.zipf_counts(B, H, S // qblk, s=c["zipf_s"], lo=1, hi=c["max_blocks"], seed=seed + 3)
+    bi, bc = (t.to(dev) for t in wl.ragged_block_lists(B, H, S, qblk, 64, cnt, seed=seed + 4))
+    o = torch.empty_like(q)
+    order = torch.empty((bc.numel(),), dtype=torch.int32, device=dev)
+    flops = 4.0 * float(cnt.sum()) * qblk * 64 * D
+    ms0, _ = time_steps(lambda: capi.sp_attn_blocks(o, q, k, v, bi, bc, qblk=qblk), steps, warmup)
+    ms_o, _ = time_steps(lambda: capi.qblock_order(order, bc), steps, warmup)
+
+    def ordered():
+        capi.qblock_order(order, bc)
+        capi.sp_attn_blocks(o, q, k, v, bi, bc, qblk=qblk, order=order)
+
+    ms1, _ = time_steps(ordered, steps, warmup)
+    return dict(ms_default=ms0, ms_ordered=ms1, ms_order_kernel=ms_o, flops=flops, kept_blocks=int(cnt.sum()))
+
+
 def bench_compaction(dev, steps, warmup, seed=0):
     """booleanmask_to_indexmask at the padded threshold workload: B=1, H=24, N=32760 -> mask
     [1,24,256,32768] int32 with ~8 % of the entries set."""
@@ -250,7 +272,7 @@ def main(argv=None) -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-extras", action="store_true", help="only the headline kernel")
-    ap.add_argument("--only", default="", help="run one leg only: sparse|tokens|compact|dense|sweeps|copy|packed|topk (no JSON contract)")
+    ap.add_argument("--only", default="", help="run one leg only: sparse|tokens|compact|dense|sweeps|copy|packed|topk|zipf (no JSON contract)")
     args = ap.parse_args(argv)
     if args.gpus != 1:
         print("bench.py: this library is single-GPU; run with --gpus 1 (got %d)" % args.gpus, file=sys.stderr)
@@ -264,7 +286,7 @@ def main(argv=None) -> int:
 
     if args.only:
         fn = {"sparse": bench_sparse, "compact": bench_compaction, "dense": bench_dense, "sweeps": bench_sweeps,
-              "copy": bench_copy, "packed": bench_packed, "tokens": bench_tokens, "topk": bench_topk}[args.only]
+              "copy": bench_copy, "packed": bench_packed, "tokens": bench_tokens, "topk": bench_topk, "zipf": bench_zipf}[args.only]
         r = fn(dev, args.steps, args.warmup)
         r.pop("tensors", None)
         print(json.dumps(r))
@@ -291,6 +313,12 @@ def main(argv=None) -> int:
                               "kernel": "attn_fwd_kernel<128,64,KV_TOKENS>", "ms": tk["ms"],
                               "tflops": tk["flops"] / (tk["ms"] * 1e-3) / 1e12,
                               "mfma_frac": tk["flops"] / (tk["ms"] * 1e-3) / 1e12 / PEAK_BF16_TFLOPS}
+        zp = bench_zipf(dev, max(2, args.steps // 4), 2)
+        out["zipf_lists"] = {"workload": "cfg5: B=1 H=8 N=65536 d=128, q-block 128, Zipf(1.2) block counts in [1,1024]",
+                             "ms_default_order": zp["ms_default"], "ms_longest_first": zp["ms_ordered"],
+                             "order_kernel_ms": zp["ms_order_kernel"],
+                             "tflops_longest_first": zp["flops"] / zp["ms_ordered"] / 1e9,
+                             "mfma_frac_longest_first": zp["flops"] / zp["ms_ordered"] / 1e9 / PEAK_BF16_TFLOPS}
         cp = bench_compaction(dev, args.steps, args.warmup)
         gbps = cp["bytes"] / (cp["ms"] * 1e-3) / 1e9
         out["mask_pass"] = {"kernel": "compact_kernel (booleanmask_to_indexmask)", "workload": "cfg4 mask %s int32, %.1f%% kept"

@@ -30,6 +30,9 @@ _SIGNATURES = {
     "spattn_full_attn": (_c_int, [_c_void_p] * 5 + [_c_int] * 5 + [_c_float, _c_void_p]),
     "spattn_sp_attn": (_c_int, [_c_void_p] * 7 + [_c_int] * 7 + [_c_float, _c_void_p]),
     "spattn_sp_attn_blocks": (_c_int, [_c_void_p] * 7 + [_c_int] * 7 + [_c_float, _c_void_p]),
+    "spattn_sp_attn_ordered": (_c_int, [_c_void_p] * 8 + [_c_int] * 7 + [_c_float, _c_void_p]),
+    "spattn_sp_attn_blocks_ordered": (_c_int, [_c_void_p] * 8 + [_c_int] * 7 + [_c_float, _c_void_p]),
+    "spattn_qblock_order": (_c_int, [_c_void_p] * 2 + [_c_int, _c_void_p]),
     "spattn_all_index_mask": (_c_int, [_c_void_p] * 2 + [_c_int] * 5 + [_c_void_p]),
     "spattn_fullattn_maxq_denom": (_c_int, [_c_void_p] * 6 + [_c_int] * 5 + [_c_float, _c_void_p]),
     "spattn_maxq_denom": (_c_int, [_c_void_p] * 4 + [_c_int] * 5 + [_c_float, _c_void_p]),
@@ -112,8 +115,11 @@ def full_attn(o, q, k, v, *, lse=None, kv_len=0, scale=0.0, stream=None):
                                    B, H, S, D, kv_len, scale, _stream(stream)))
 
 
-def sp_attn(o, q, k, v, kv_indices, kv_num_indices, *, lse=None, qblk=None, kv_len=0, scale=0.0, stream=None):
-    """Token-list sparse attention.  qblk defaults to the value implied by kv_indices.shape[2]."""
+def sp_attn(o, q, k, v, kv_indices, kv_num_indices, *, lse=None, qblk=None, kv_len=0, scale=0.0, order=None,
+            stream=None):
+    """Token-list sparse attention.  qblk defaults to the value implied by kv_indices.shape[2].
+    order: optional int32 [B*H*SB] work order from qblock_order (same results, better balance
+    when the lists differ much in length)."""
     B, H, S, D = _bhsd(q)
     if kv_indices.dim() != 4:
         raise ValueError("kv_indices must be [B,H,SB,mask_stride]")
@@ -121,13 +127,21 @@ def sp_attn(o, q, k, v, kv_indices, kv_num_indices, *, lse=None, qblk=None, kv_l
         qblk = infer_qblk(S, int(kv_indices.shape[2]))
     if kv_num_indices.numel() != B * H * int(kv_indices.shape[2]):
         raise ValueError("kv_num_indices must have B*H*SB entries")
-    _check(load().spattn_sp_attn(_ptr(o, bf16), _ptr(lse, f32), _ptr(q, bf16), _ptr(k, bf16), _ptr(v, bf16),
-                                 _ptr(kv_indices, i32), _ptr(kv_num_indices, i32), int(kv_indices.shape[3]), qblk,
-                                 B, H, S, D, kv_len, scale, _stream(stream)))
+    if order is None:
+        _check(load().spattn_sp_attn(_ptr(o, bf16), _ptr(lse, f32), _ptr(q, bf16), _ptr(k, bf16), _ptr(v, bf16),
+                                     _ptr(kv_indices, i32), _ptr(kv_num_indices, i32), int(kv_indices.shape[3]), qblk,
+                                     B, H, S, D, kv_len, scale, _stream(stream)))
+        return
+    if order.numel() != kv_num_indices.numel():
+        raise ValueError("order must have B*H*SB entries")
+    _check(load().spattn_sp_attn_ordered(_ptr(o, bf16), _ptr(lse, f32), _ptr(q, bf16), _ptr(k, bf16), _ptr(v, bf16),
+                                         _ptr(kv_indices, i32), _ptr(kv_num_indices, i32), _ptr(order, i32),
+                                         int(kv_indices.shape[3]), qblk, B, H, S, D, kv_len, scale, _stream(stream)))
 
 
-def sp_attn_blocks(o, q, k, v, blk_indices, blk_counts, *, lse=None, qblk=None, kv_len=0, scale=0.0, stream=None):
-    """Block-list sparse attention over 64-key blocks."""
+def sp_attn_blocks(o, q, k, v, blk_indices, blk_counts, *, lse=None, qblk=None, kv_len=0, scale=0.0, order=None,
+                   stream=None):
+    """Block-list sparse attention over 64-key blocks.  order: as for sp_attn."""
     B, H, S, D = _bhsd(q)
     if blk_indices.dim() != 4:
         raise ValueError("blk_indices must be [B,H,SB,max_blocks]")
@@ -135,9 +149,25 @@ def sp_attn_blocks(o, q, k, v, blk_indices, blk_counts, *, lse=None, qblk=None, 
         qblk = infer_qblk(S, int(blk_indices.shape[2]))
     if blk_counts.numel() != B * H * int(blk_indices.shape[2]):
         raise ValueError("blk_counts must have B*H*SB entries")
-    _check(load().spattn_sp_attn_blocks(_ptr(o, bf16), _ptr(lse, f32), _ptr(q, bf16), _ptr(k, bf16), _ptr(v, bf16),
-                                        _ptr(blk_indices, i32), _ptr(blk_counts, i32), int(blk_indices.shape[3]),
-                                        qblk, B, H, S, D, kv_len, scale, _stream(stream)))
+    if order is None:
+        _check(load().spattn_sp_attn_blocks(_ptr(o, bf16), _ptr(lse, f32), _ptr(q, bf16), _ptr(k, bf16), _ptr(v, bf16),
+                                            _ptr(blk_indices, i32), _ptr(blk_counts, i32), int(blk_indices.shape[3]),
+                                            qblk, B, H, S, D, kv_len, scale, _stream(stream)))
+        return
+    if order.numel() != blk_counts.numel():
+        raise ValueError("order must have B*H*SB entries")
+    _check(load().spattn_sp_attn_blocks_ordered(_ptr(o, bf16), _ptr(lse, f32), _ptr(q, bf16), _ptr(k, bf16),
+                                                _ptr(v, bf16), _ptr(blk_indices, i32), _ptr(blk_counts, i32),
+                                                _ptr(order, i32), int(blk_indices.shape[3]), qblk, B, H, S, D, kv_len,
+                                                scale, _stream(stream)))
+
+
+def qblock_order(order, counts, *, stream=None):
+    """order: int32 [n] <- the q-blocks (flat indices of counts) longest list first; lists within
+    a factor of two of each other keep the default order."""
+    if order.numel() != counts.numel():
+        raise ValueError("order and counts must have the same number of entries")
+    _check(load().spattn_qblock_order(_ptr(order, i32), _ptr(counts, i32), int(counts.numel()), _stream(stream)))
 
 
 def all_index_mask(kv_indices, kv_num_indices, batch, heads, seqblocks, seq, *, stream=None):

@@ -94,7 +94,9 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   const int ksub = wave / NQW;
 
   const int total = p.nqblk * p.H * p.B;
-  const int wg = xcd_remap(blockIdx.x, total);
+  // a caller-given work order (longest lists first) replaces the XCD-contiguous default
+  const int wg = p.order ? ((const __attribute__((address_space(4))) int*)p.order)[blockIdx.x]
+                         : xcd_remap(blockIdx.x, total);
   const int qb = wg % p.nqblk;
   const int bh = wg / p.nqblk;
 

@@ -180,6 +180,46 @@ int spattn_qk_topkmask_indices(int* kv_indices, int* num_kv_indices, void* score
                                         score_stride, idx_stride, as_stream(stream)));
 }
 
+int spattn_qblock_order(int* order, const int* counts, int n, void* stream) {
+  if (!order || !counts) return done(SPATTN_ERR_NULL);
+  if (n <= 0) return done(SPATTN_ERR_SHAPE);
+  return from_hip(spattn::run_qblock_order(order, counts, n, as_stream(stream)));
+}
+
+int spattn_sp_attn_ordered(void* o, float* lse, const void* q, const void* k, const void* v, const int* kv_indices,
+                           const int* num_kv_indices, const int* order, int mask_stride, int qblk, int B, int H, int S,
+                           int D, int kv_len, float scale, void* stream) {
+  if (int st = check_qkv(q, k, B, H, S, D)) return done(st);
+  if (!o || !v || !kv_indices || !num_kv_indices || !order) return done(SPATTN_ERR_NULL);
+  if (misaligned(o) || misaligned(v) || misaligned(kv_indices)) return done(SPATTN_ERR_ALIGN);
+  if (qblk != 64 && qblk != 128) return done(SPATTN_ERR_QBLK);
+  if (mask_stride <= 0 || mask_stride % 128 != 0) return done(SPATTN_ERR_STRIDE);
+  spattn::AttnParams p = base_params(q, k, v, o, B, H, S, D, kv_len, scale, qblk);
+  p.lse = lse;
+  p.idx = kv_indices;
+  p.cnt = num_kv_indices;
+  p.idx_stride = mask_stride;
+  p.order = order;
+  return from_hip(spattn::run_attn_tokens(p, D, qblk, as_stream(stream)));
+}
+
+int spattn_sp_attn_blocks_ordered(void* o, float* lse, const void* q, const void* k, const void* v,
+                                  const int* blk_indices, const int* blk_counts, const int* order, int max_blocks,
+                                  int qblk, int B, int H, int S, int D, int kv_len, float scale, void* stream) {
+  if (int st = check_qkv(q, k, B, H, S, D)) return done(st);
+  if (!o || !v || !blk_indices || !blk_counts || !order) return done(SPATTN_ERR_NULL);
+  if (misaligned(o) || misaligned(v)) return done(SPATTN_ERR_ALIGN);
+  if (qblk != 64 && qblk != 128) return done(SPATTN_ERR_QBLK);
+  if (max_blocks <= 0) return done(SPATTN_ERR_SHAPE);
+  spattn::AttnParams p = base_params(q, k, v, o, B, H, S, D, kv_len, scale, qblk);
+  p.lse = lse;
+  p.idx = blk_indices;
+  p.cnt = blk_counts;
+  p.idx_stride = max_blocks;
+  p.order = order;
+  return from_hip(spattn::run_attn_blocks(p, D, qblk, as_stream(stream)));
+}
+
 // ---- the reference's binding surface: default stream, default scale, q-block 128 ----
 
 void attn_fwd_wg_impl(void* o, void* q, void* k, void* v, int batch, int heads, int seq, int D) {

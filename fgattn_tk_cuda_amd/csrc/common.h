@@ -35,6 +35,7 @@ struct AttnParams {
   const int* idx;     // [B,H,SBq,idx_stride] token ids or block ids
   const int* cnt;     // [B*H*SBq]
   int idx_stride;
+  const int* order;   // optional [B*H*nqblk]: the q-block (flat index) that workgroup i takes
   int B, H, S;
   int kv_len;         // keys with row >= kv_len never contribute
   int Sp;             // row stride of max_q / denom

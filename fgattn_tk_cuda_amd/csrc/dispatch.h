@@ -27,4 +27,7 @@ hipError_t run_topk_mask(int* kv_indices, int* kv_num, uint16_t* score, uint16_t
                          const uint16_t* k, int B, int H, int S, int D, int blk, int kv_len, int select_k,
                          int score_stride, int idx_stride, hipStream_t stream);
 
+// order_kernels.hip
+hipError_t run_qblock_order(int* order, const int* counts, int n, hipStream_t stream);
+
 }  // namespace spattn

@@ -88,9 +88,17 @@ void sp_attn(torch::Tensor o, torch::Tensor q, torch::Tensor k, torch::Tensor v,
   // the reference does not check the shape of kv_num_indices, only its element order
   TORCH_CHECK(kv_num_indices.numel() == q.size(0) * q.size(1) * kv_indices.size(2), "kv_num_indices must have B*H*SB entries");
   const DeviceGuard guard(q.device());
-  check_status(spattn_sp_attn(o.data_ptr(), nullptr, q.data_ptr(), k.data_ptr(), v.data_ptr(), kv_indices.data_ptr<int>(),
-                              kv_num_indices.data_ptr<int>(), (int)kv_indices.size(3), qblk, (int)q.size(0),
-                              (int)q.size(1), (int)q.size(2), (int)q.size(3), 0, 0.f, cur_stream()),
+  // Threshold masks give lists of very different lengths: the q-blocks are handed to the
+  // workgroups longest list first (the order is a small device tensor from torch's caching
+  // allocator; lists within a factor of two of each other keep the default order).
+  torch::Tensor order = torch::empty({kv_num_indices.numel()}, kv_num_indices.options());
+  check_status(spattn_qblock_order(order.data_ptr<int>(), kv_num_indices.data_ptr<int>(), (int)kv_num_indices.numel(),
+                                   cur_stream()),
+               "sp_attn (work order)");
+  check_status(spattn_sp_attn_ordered(o.data_ptr(), nullptr, q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                      kv_indices.data_ptr<int>(), kv_num_indices.data_ptr<int>(), order.data_ptr<int>(),
+                                      (int)kv_indices.size(3), qblk, (int)q.size(0), (int)q.size(1), (int)q.size(2),
+                                      (int)q.size(3), 0, 0.f, cur_stream()),
                "sp_attn");
 }
 

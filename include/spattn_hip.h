@@ -134,6 +134,21 @@ int spattn_qk_topkmask_indices(int* kv_indices, int* num_kv_indices, void* score
                                const void* k, int batch, int heads, int seq, int D, int blocksz, int kv_len,
                                int select_k, int score_stride, int idx_stride, void* stream);
 
+/* Work order for lists of very uneven length.  No counterpart in the reference, whose grid is
+ * fixed to (q-block, head, batch) (include/sparseattn_asyncgatherload_padded.cuh:273).
+ * spattn_qblock_order writes into order[0..n) a permutation of 0..n-1 (n = batch*heads*SB, the
+ * flat q-block index of the count tensor): longest lists first, in quarter-octave classes of the
+ * count, stable inside a class; if the longest list is less than twice the shortest, the default order.  The
+ * _ordered forms of the two list-driven attention entry points let workgroup i take q-block
+ * order[i]; results are bit-identical to the plain forms, only the schedule changes. */
+int spattn_qblock_order(int* order, const int* counts, int n, void* stream);
+int spattn_sp_attn_ordered(void* o, float* lse, const void* q, const void* k, const void* v, const int* kv_indices,
+                           const int* num_kv_indices, const int* order, int mask_stride, int qblk, int batch, int heads,
+                           int seq, int D, int kv_len, float scale, void* stream);
+int spattn_sp_attn_blocks_ordered(void* o, float* lse, const void* q, const void* k, const void* v,
+                                  const int* blk_indices, const int* blk_counts, const int* order, int max_blocks,
+                                  int qblk, int batch, int heads, int seq, int D, int kv_len, float scale, void* stream);
+
 /* Status of the most recent call on this host thread, and its text. */
 int spattn_last_status(void);
 const char* spattn_status_string(int status);

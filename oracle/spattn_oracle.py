@@ -346,3 +346,33 @@ def topk_select(score, select_k: int, kv_len: int | None = None):
         order = np.lexsort((np.arange(kv_len), -row))   # by score descending, then key ascending
         out[i] = np.sort(order[:kk])
     return out.reshape(*score.shape[:-1], kk)
+
+
+def _xcd_remap(i, n, xcds=8):
+    per = n // xcds
+    lim = per * xcds
+    return np.where(i >= lim, i, (i % xcds) * per + i // xcds)
+
+
+def qblock_order(counts, sub_bits: int = 2, octaves: int = 22):
+    """Work order of the list-driven attention kernels (no counterpart in the reference, whose
+    grid is fixed, include/sparseattn_asyncgatherload_padded.cuh:273): q-blocks by list length,
+    longest first, in quarter-octave classes of the count (the leading one and the two bits
+    below it), stable inside a class; if the longest list is less than twice the shortest the default order is kept
+    (neighbouring q-blocks together on one XCD).
+    Integer work; pinned by its defining properties (a permutation, class-monotone, stable) and
+    by a brute-force sort in the tests."""
+    c = np.asarray(counts).reshape(-1).astype(np.int64)
+    n = c.size
+    lo, hi = int(c.min()), int(c.max())
+    if hi <= 0 or hi < 2 * lo:
+        return _xcd_remap(np.arange(n), n).astype(np.int32)
+    classes = (octaves << sub_bits) + 2
+    lg = np.zeros(n, np.int64)
+    pos = c > 0
+    lg[pos] = np.frexp(c[pos].astype(np.float64))[1] - 1      # floor(log2 c), exact below 2^53
+    m = (1 << sub_bits) - 1
+    below = np.where(lg >= sub_bits, (c >> np.maximum(lg - sub_bits, 0)) & m, (c << np.maximum(sub_bits - lg, 0)) & m)
+    fine = np.minimum((lg << sub_bits) + below, classes - 2)
+    cls = np.where(pos, classes - 2 - fine, classes - 1)
+    return np.argsort(cls, kind="stable").astype(np.int32)

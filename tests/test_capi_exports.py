@@ -22,7 +22,7 @@ def test_header_declares_expected_surface():
     for ref in ("attn_fwd_wg_impl", "attn_sparse_fwd_wg_impl", "allindex_mask_impl", "attn_maxq_denom_impl",
                 "maxq_denom_impl", "booleanmask_128_impl", "booleanmask_to_indexmask_impl"):
         assert ref in names
-    assert "spattn_sp_attn_blocks" in names and "spattn_packedmask_to_indexmask" in names and "spattn_qk_topkmask_indices" in names and len(names) == 21
+    assert "spattn_sp_attn_blocks" in names and "spattn_packedmask_to_indexmask" in names and "spattn_qk_topkmask_indices" in names and "spattn_qblock_order" in names and len(names) == 24
 
 
 def test_library_exports_every_declared_symbol():

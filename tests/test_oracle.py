@@ -291,3 +291,33 @@ def test_cfg1_plumbing_case_oracle_equals_dense_masked_softmax():
         s = (q[0, h] @ k[0, h].T) * D ** -0.5
         s.masked_fill_(~cma.block_mask_rows(bi[0, h], bc[0, h], 0, S, qblk, kvblk, S), float("-inf"))
         assert np.abs(lse[0, h] - torch.logsumexp(s, -1).numpy()).max() < 2e-5
+
+
+def test_qblock_order_is_a_stable_class_sort():
+    """Longest lists first in quarter-octave classes, stable inside a class; lists within a factor
+    of two of each other keep the XCD-contiguous default order.  Checked against a pure-Python sort."""
+    rng = np.random.default_rng(0)
+
+    def cls(x):
+        if x <= 0:
+            return 89
+        lg = x.bit_length() - 1
+        below = ((x >> (lg - 2)) & 3) if lg >= 2 else ((x << (2 - lg)) & 3)
+        return 88 - min(4 * lg + below, 88)
+
+    for trial in range(200):
+        n = int(rng.integers(1, 300))
+        c = rng.integers(0, 5000, size=n)
+        if trial % 5 == 0:
+            c = c // 1000
+        got = orc.qblock_order(c)
+        assert sorted(got.tolist()) == list(range(n))
+        lo, hi = int(c.min()), int(c.max())
+        if hi <= 0 or hi < 2 * lo:
+            assert got.tolist() == orc._xcd_remap(np.arange(n), n).tolist()
+            continue
+        assert got.tolist() == sorted(range(n), key=lambda i: (cls(int(c[i])), i))
+    # equal lengths: the default order, every XCD a contiguous range
+    d = orc.qblock_order(np.full(32, 7))
+    assert d[:8].tolist() == [0, 4, 8, 12, 16, 20, 24, 28] and sorted(d.tolist()) == list(range(32))
+    assert orc.qblock_order(np.array([1 << 30, 3, 1 << 24, 0])).tolist() == [0, 2, 1, 3]
