@@ -359,8 +359,8 @@ __global__ __launch_bounds__(256) void topk_select_kernel(int* __restrict__ kv_i
 // (kv_len <= kTopkLdsMaxKeys); longer rows take topk_select_kernel.
 constexpr int kTopkLdsMaxKeys = 72000;
 // A score row has few distinct exponents: most keys of a pass land in a handful of bins.  Every
-// bin is therefore kept as 16 partial counts, one per lane & 15, next to each other (16
-// different banks): a wave's adds to one bin meet 4 to an address instead of 64.
+// bin is therefore kept as 4 partial counts, one per lane & 3, next to each other (4
+// different banks): the adds of a wave to one bin meet 16 to an address instead of 64.
 constexpr int kTopkSubs = 4;
 constexpr int kTopkThreads = 512;
 constexpr int kTopkWaves = kTopkThreads / 64;
