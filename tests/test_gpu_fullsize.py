@@ -123,6 +123,66 @@ def test_cfg5_zipf_lists(dev):
         assert_close_stat(f32(lse[0, h, r]), wlse, "zipf lse")
 
 
+def test_cfg5_full_size_work_order_changes_nothing(dev):
+    """B=1 H=8 N=65536 d=128, 128-row q-blocks, Zipf(1.2) counts in [1,1024]: the longest-first
+    work order gives bit-identical O and lse; sampled q-blocks against the oracle."""
+    print("case cfg5 full size, ordered", flush=True)
+    c = wl.CONFIGS["cfg5_zipf_64k"]
+    B, H, S, D, qblk = c["B"], c["H"], c["S"], c["D"], c["qblk"]
+    q, k, v = wl.randn_qkv(B, H, S, D, seed=14)
+    counts = wl.zipf_counts(B, H, S // qblk, s=c["zipf_s"], lo=1, hi=c["max_blocks"], seed=15)
+    bi, bc = wl.ragged_block_lists(B, H, S, qblk, 64, counts, seed=16)
+    qd, kd, vd, bid, bcd = to_dev(dev, q, k, v, bi, bc)
+    o1, o2 = torch.empty_like(qd), torch.empty_like(qd)
+    l1 = torch.empty((B, H, S), device=dev)
+    l2 = torch.empty((B, H, S), device=dev)
+    order = torch.empty((bcd.numel(),), dtype=torch.int32, device=dev)
+    capi.qblock_order(order, bcd)
+    capi.sp_attn_blocks(o1, qd, kd, vd, bid, bcd, lse=l1, qblk=qblk)
+    capi.sp_attn_blocks(o2, qd, kd, vd, bid, bcd, lse=l2, qblk=qblk, order=order)
+    torch.cuda.synchronize()
+    assert np.array_equal(order.cpu().numpy(), orc.qblock_order(counts))
+    assert torch.equal(o1, o2) and torch.equal(l1, l2)
+    flat = np.argsort(counts.reshape(-1))
+    for pick in (flat[0], flat[-1], flat[len(flat) // 2]):
+        h, i = divmod(int(pick), S // qblk)
+        wo, wlse = _oracle_block_rows(q, k, v, bi, bc, 0, h, i, qblk, S)
+        r = slice(i * qblk, (i + 1) * qblk)
+        assert_close_o(f32(o2[0, h, r]), wo, "cfg5 q-block (%d,%d) count %d" % (h, i, counts[0, h, i]))
+        assert_close_stat(f32(l2[0, h, r]), wlse, "cfg5 lse")
+
+
+def test_cfg4_shape_topk_generator_sampled_rows(dev):
+    """The top-k mask generator at B=1 H=24 N=32760 d=64, 2621 keys per 128-row q-block: sampled
+    rows of the score matrix against the oracle, the selection of those rows bit-exact given
+    the device's scores, counts and list order everywhere."""
+    print("case cfg4 top-k", flush=True)
+    c = wl.CONFIGS["cfg4_threshold_padded"]
+    B, H, S, D = c["B"], c["H"], c["S"], c["D"]
+    q, k, _ = wl.clustered_qkv(B, H, S, D, seed=17)
+    SB, Sp, select_k = 256, 32768, int(round(c["keep"] * S))
+    stride = 128 * orc.ceil_div(select_k, 128)
+    kvi = torch.full((B, H, SB, stride), -7, dtype=torch.int32, device=dev)
+    kvn = torch.zeros((B, H, SB), dtype=torch.int32, device=dev)
+    score = torch.empty((B, H, SB, Sp), dtype=torch.bfloat16, device=dev)
+    qmean = torch.empty((B, H, SB, D), dtype=torch.bfloat16, device=dev)
+    capi.qk_topkmask_indices(kvi, kvn, score, qmean, q.to(dev), k.to(dev), select_k, blocksz=128)
+    torch.cuda.synchronize()
+    assert bool((kvn == select_k).all())
+    lists = kvi[..., :select_k]
+    assert bool((lists[..., 1:] > lists[..., :-1]).all()) and bool((lists >= 0).all()) and bool((lists < S).all())
+    assert bool((kvi[..., select_k:] == -7).all())
+    rng = np.random.default_rng(18)
+    for h, m in [(int(rng.integers(H)), int(rng.integers(SB))) for _ in range(3)] + [(H - 1, SB - 1)]:
+        want_qm, want_sc = orc.qblock_mean_scores(f32(q[:, h:h + 1, m * 128:(m + 1) * 128]), f32(k[:, h:h + 1]), 128)
+        assert np.array_equal(f32(qmean[0, h, m]), want_qm[0, 0, 0])
+        got = f32(score[0, h, m, :S])
+        diff = got != want_sc[0, 0, 0]
+        assert diff.mean() < 0.02
+        assert np.all(np.abs(got - want_sc[0, 0, 0])[diff] <= np.abs(want_sc[0, 0, 0][diff]) * 2.0 ** -7 + 1e-5)
+        assert np.array_equal(kvi[0, h, m, :select_k].cpu().numpy(), orc.topk_select(got[None], select_k)[0])
+
+
 def test_cfg4_padded_threshold_pipeline(dev):
     """N=32760 (padded to 32768), d=64, clustered keys: statistics -> vote mask -> index lists
     -> sparse attention, two heads; each stage checked on sampled q-blocks."""
