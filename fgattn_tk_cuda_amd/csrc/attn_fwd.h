@@ -267,10 +267,18 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
 #pragma unroll
     for (int j = 0; j < 3; ++j) ids_resolve(j, idr[j], idw[j], idh[j]);
   }
-  // what prepare_tile takes for tile j (a prologue tile: j < 3)
+  // What prepare_tile takes for tile j (a prologue tile: j < 3).  Block lists: the first three
+  // entries are fetched before anything depends on the count (list positions are clamped, an
+  // entry past the count is simply not used), so that the count and the entries travel
+  // together instead of one scalar-load latency after the other.
+  int hd[3] = {0, 0, 0};
+  if constexpr (MODE != KV_TOKENS) {
+#pragma unroll
+    for (int j = 0; j < 3; ++j) hd[j] = tile_desc(j);
+  }
   auto head_desc = [&](int j) -> int {
     if constexpr (MODE == KV_TOKENS) return idr[j];
-    else return tile_desc(j);
+    else return hd[j];
   };
   using G0 = std::integral_constant<int, 0>;
   using G1 = std::integral_constant<int, 1>;
@@ -640,13 +648,13 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     __syncthreads();
     qk_tile(std::false_type{}, std::false_type{}, 0, 0, s_e, s_e, nullptr, false);
     if constexpr (MODE == KV_TOKENS) mask_tile(idw[0], idh[0], s_e);
-    else mask_tile(tile_desc(0), 0, s_e);
+    else mask_tile(hd[0], 0, s_e);
     maybe_rescale(row_stats(s_e));
 
     int it = 0;
     if constexpr (MODE != KV_TOKENS) {
 #pragma unroll
-      for (int j = 1; j <= NK; ++j) idw[j] = tile_desc(j);
+      for (int j = 1; j <= NK; ++j) idw[j] = j < 3 ? hd[j] : tile_desc(j);
     }
     // Rounds of six tiles without side exits (the register allocator handles one plain
     // back-edge far better than six exits), then up to five single tiles.
@@ -691,7 +699,11 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   // ---- combine the two 32-lane halves, then the two key halves -------------------
   float l_tot = pair_sum(l_run);
   if constexpr (KSPLIT == 2) {
+    // per row half: three rows of 64 floats (reference, sum, true max), then the accumulators
+    // four registers at a time, 16 bytes per lane
     float* mg = reinterpret_cast<float*>(smem) + qsub * ((HAS_V ? D / 2 : 0) + 3) * 64;
+    typedef __attribute__((ext_vector_type(4))) float f32x4;
+    f32x4* mg4 = reinterpret_cast<f32x4*>(mg + 3 * 64);
     if (ksub == 1) {
       mg[lane] = mr_sf;
       mg[64 + lane] = l_tot;
@@ -700,7 +712,10 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
 #pragma unroll
         for (int db = 0; db < NDB; ++db)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) mg[(3 + db * 16 + r) * 64 + lane] = oacc[db][r];
+          for (int j = 0; j < 4; ++j) {
+            const f32x4 x = {oacc[db][4 * j], oacc[db][4 * j + 1], oacc[db][4 * j + 2], oacc[db][4 * j + 3]};
+            mg4[(db * 4 + j) * 64 + lane] = x;
+          }
       }
     }
     __syncthreads();
@@ -717,7 +732,11 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
 #pragma unroll
       for (int db = 0; db < NDB; ++db)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) oacc[db][r] = oacc[db][r] * a1 + mg[(3 + db * 16 + r) * 64 + lane] * a2;
+        for (int j = 0; j < 4; ++j) {
+          const f32x4 x = mg4[(db * 4 + j) * 64 + lane];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) oacc[db][4 * j + i] = oacc[db][4 * j + i] * a1 + x[i] * a2;
+        }
     }
   }
 
