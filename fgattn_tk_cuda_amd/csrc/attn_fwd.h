@@ -326,7 +326,14 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
 
-  u32x4 pb[HAS_V ? 2 * NMB : 1];   // P^T operands, k-step 2mb + h
+  // SPLIT_SM: the exponentials of a tile are taken in two halves, score registers 0-7 of every
+  // block under the P V multiplies of the tile before, registers 8-15 under the QK^T multiplies
+  // of the tile after, so that every multiply has the same vector-ALU work next to it (all of
+  // it under QK^T leaves the vector ALU the bottleneck there and idle under P V).  Needs the
+  // reference fixed before the tile's scores exist, which LAZY_MAX gives.
+  // (at d=128 a wave of a 128-row q-block has no registers left for the second set of operands)
+  constexpr bool SPLIT_SM = LAZY_MAX && HAS_V && (D == 64 || QBLK == 64);
+  u32x4 pb[SPLIT_SM ? 2 : 1][HAS_V ? 2 * NMB : 1];   // P^T operands, k-step 2mb + h; SPLIT_SM: by tile parity
 
   // Per-lane LDS addresses inside slot 0; slot, score block and k-step offsets are added
   // as constants (instruction immediates in the unrolled loop).
@@ -432,38 +439,44 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   // p = exp2(s*sf - reference) for registers r0..r0+cnt-1 of block mb; adds to the row sum
   // and leaves P^T as bf16 MFMA operands (k-step 2mb+h takes registers 8h..8h+7 of block
   // mb, i.e. keys 32mb + 16h + {4g..4g+3} and 32mb + 16h + 8 + {4g..4g+3}).
-  auto softmax_chunk = [&](f32x16 (&s)[NMB], float base, int mb, int r0, int cnt) {
+  auto softmax_chunk = [&](const f32x16 (&s)[NMB], float base, int mb, int r0, int cnt, int par) {
 #pragma unroll
     for (int r = r0; r < r0 + cnt; r += 2) {
       const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[mb][r], p.sf, -base));
       const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[mb][r + 1], p.sf, -base));
       l_tile = (mb == 0 && r == 0) ? e0 : l_tile + e0;
       l_tile += e1;
-      if constexpr (HAS_V) pb[2 * mb + (r >> 3)][(r & 7) >> 1] = pack_bf16(e0, e1);
+      if constexpr (HAS_V) pb[SPLIT_SM ? par : 0][2 * mb + (r >> 3)][(r & 7) >> 1] = pack_bf16(e0, e1);
     }
   };
   // Pin the softmax results where they are produced; otherwise the compiler sinks the
   // whole softmax to the first use of P and nothing overlaps the MFMAs.
-  auto pin_softmax = [&]() {
+  // half: 0 = the operands of registers 0-7, 1 = of registers 8-15, 2 = both
+  auto pin_softmax = [&](int par, int half) {
     asm volatile("" : "+v"(l_tile));
     if constexpr (HAS_V) {
 #pragma unroll
       for (int ks = 0; ks < 2 * NMB; ++ks)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(pb[ks][i]));
+        for (int i = 0; i < 4; ++i)
+          if (half == 2 || (ks & 1) == half) asm volatile("" : "+v"(pb[SPLIT_SM ? par : 0][ks][i]));
     }
   };
-  auto softmax_only = [&](f32x16 (&s)[NMB]) {
+  auto softmax_only = [&](const f32x16 (&s)[NMB], int par) {
 #pragma unroll
-    for (int mb = 0; mb < NMB; ++mb) softmax_chunk(s, base_eff, mb, 0, 16);
+    for (int mb = 0; mb < NMB; ++mb) softmax_chunk(s, base_eff, mb, 0, 16, par);
+  };
+  auto softmax_half = [&](const f32x16 (&s)[NMB], int par, int half) {
+#pragma unroll
+    for (int mb = 0; mb < NMB; ++mb) softmax_chunk(s, base_eff, mb, 8 * half, 8, par);
   };
   // Closes the softmax of a tile: adds its sum to the denominator.  LAZY_MAX: first redoes
   // the tile against a new reference if some row of the wave outgrew the old one.
-  auto softmax_close = [&](f32x16 (&s)[NMB]) {
+  auto softmax_close = [&](const f32x16 (&s)[NMB], int par) {
     if constexpr (LAZY_MAX) {
       if (__any(!(l_tile <= kTrigger))) {
         maybe_rescale(row_stats(s));
-        softmax_only(s);
+        softmax_only(s, par);
       }
     }
     l_run += l_tile;
@@ -494,10 +507,11 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   // so that PV does not start by waiting for LDS.
   constexpr int kEarly = 1;
   auto qk_tile = [&](auto with_sm, auto early_v, uint32_t kofs, uint32_t vofs, f32x16 (&s_out)[NMB], f32x16 (&s_in)[NMB],
-                     const TileLoad* tl, bool live) {
+                     int par_in, const TileLoad* tl, bool live) {
     constexpr bool WITH_SM = decltype(with_sm)::value;
     constexpr bool EARLY_V = decltype(early_v)::value;
     constexpr int EPM = 16 / NT;
+    constexpr int MPP = NT / 4;   // SPLIT_SM: multiplies per pair of score registers 8-15
     const float base = base_eff;
 #pragma unroll
     for (int mb = 0; mb < NMB; ++mb) {
@@ -514,7 +528,11 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
 #pragma unroll
         for (int t = t0; t < t1; ++t) {
           s_out[mb] = mfma32(ka[t], qf[t], t == 0 ? zero : s_out[mb]);
-          if constexpr (WITH_SM) softmax_chunk(s_in, base, mb, t * EPM, EPM);
+          if constexpr (WITH_SM && SPLIT_SM) {
+            if (t % MPP == 0) softmax_chunk(s_in, base, mb, 8 + 2 * (t / MPP), 2, par_in);
+          } else if constexpr (WITH_SM) {
+            softmax_chunk(s_in, base, mb, t * EPM, EPM, par_in);
+          }
           if (tl != nullptr && live) {
             constexpr int STEP = (NMB * NT) / LPT;
             const int m = mb * NT + t;
@@ -525,7 +543,11 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
 #pragma unroll
           for (int t = t0; t < t1; ++t) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);            // one MFMA
-            __builtin_amdgcn_sched_group_barrier(0x002, EPM * 7 / 2, 0);  // its share of the softmax
+            // its share of the softmax: seven instructions per pair of score registers
+            if constexpr (!SPLIT_SM) __builtin_amdgcn_sched_group_barrier(0x002, EPM * 7 / 2, 0);
+            else if constexpr (MPP == 1) __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);
+            else if (t % 2 == 0) __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+            else __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
           }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -541,14 +563,20 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
         steps(NT / 4, NT);
       }
     }
-    if constexpr (WITH_SM) pin_softmax();
+    if constexpr (WITH_SM) pin_softmax(par_in, SPLIT_SM ? 1 : 2);
   };
   // O^T += V^T P^T from the V tile at offset vofs from the first V slot, one 16-key step (NDB multiplies) at
   // a time; the operands of step 0 are in flight or here already (FIRST_LOADED), those of
   // step gi+1 are requested before step gi is multiplied.  STAT: the row maxima of s_next
   // are reduced between the multiplies; returns them (times sf).
-  auto pv_tile = [&](auto first_loaded, auto stat_c, uint32_t vofs, const TileLoad* tl, bool live, const f32x16 (&s_next)[NMB]) -> float {
+  // EARLY_SM: the exponentials of registers 0-7 of s_next (the tile after, parity par ^ 1) are
+  // taken between the multiplies.
+  auto pv_tile = [&](auto first_loaded, auto stat_c, uint32_t vofs, const TileLoad* tl, bool live, const f32x16 (&s_next)[NMB],
+                     int par, auto early_sm) -> float {
     constexpr bool STAT = decltype(stat_c)::value;
+    constexpr bool EARLY_SM = decltype(early_sm)::value;
+    constexpr int MPP = NDB / 2;   // EARLY_SM: multiplies per pair of score registers
+    const float base = base_eff;
     float mloc = 0.f;
     if constexpr (HAS_V) {
       if constexpr (!decltype(first_loaded)::value) v_reads(vofs, 0);
@@ -559,8 +587,11 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
 #pragma unroll
         for (int db = 0; db < NDB; ++db) {
           const u32x4 a = {va[gi & 1][db][0][0], va[gi & 1][db][0][1], va[gi & 1][db][1][0], va[gi & 1][db][1][1]};
-          oacc[db] = mfma32(a, pb[gi], oacc[db]);
+          oacc[db] = mfma32(a, pb[SPLIT_SM ? par : 0][gi], oacc[db]);
           const int m = gi * NDB + db;
+          if constexpr (EARLY_SM) {
+            if (m % MPP == 0) softmax_chunk(s_next, base, (m / MPP) / 4, 2 * ((m / MPP) % 4), 2, par ^ 1);
+          }
           if constexpr (STAT) {
             constexpr int PPM = (NP + NG * NDB - 1) / (NG * NDB);   // pieces per multiply
 #pragma unroll
@@ -571,8 +602,18 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
             if (m % STEP == STEP - 1) load_part(*tl, m / STEP);
           }
         }
+        if constexpr (EARLY_SM) {
+#pragma unroll
+          for (int db = 0; db < NDB; ++db) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if constexpr (MPP == 1) __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);
+            else if (db % 2 == 0) __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+            else __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+          }
+        }
         __builtin_amdgcn_sched_barrier(0);
       }
+      if constexpr (EARLY_SM) pin_softmax(par ^ 1, 0);
     } else if constexpr (STAT) {
 #pragma unroll
       for (int k = 0; k < NP; ++k) stat_piece(s_next, k, mloc);
@@ -613,22 +654,24 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     using GK = std::integral_constant<int, (KC + NK) % 3>;    // tile it+NK
     using GV = std::integral_constant<int, (KC + 1) % 3>;     // tile it+1
     const TileLoad tl_first = K_FIRST ? prepare_tile(d_k, KN, false, GK{}) : prepare_tile(d_v, VN, true, GV{});
-    qk_tile(std::true_type{}, std::integral_constant<bool, HAS_V>{}, KS * TILE, VS * TILE, s_b, s_a, &tl_first,
+    constexpr int PAR = KC & 1;
+    qk_tile(std::true_type{}, std::integral_constant<bool, HAS_V>{}, KS * TILE, VS * TILE, s_b, s_a, PAR, &tl_first,
             K_FIRST ? has_kn : true);
     // ids of tile it+NK+1: between the copies of V(it+1) and K(it+NK) in the order of issue.
     // Issued whether or not that tile exists (the position is clamped to the list): the wait
     // counts stay the same on every tile, and the registers are held until the final wait.
     if constexpr (MODE == KV_TOKENS) ids_load(it + NK + 1, idr[(KC + NK + 1) % 6]);
-    softmax_close(s_a);
+    softmax_close(s_a, PAR);
     mask_tile(m_lo, m_hi, s_b);
     if constexpr (MODE != KV_TOKENS) idw[(KC + NK + 1) % 6] = tile_desc(it + NK + 1);
     float mloc_sf;
     using stat_t = std::integral_constant<bool, !LAZY_MAX>;
     if constexpr (HAS_V) {
       const TileLoad tl_second = K_FIRST ? prepare_tile(d_v, VN, true, GV{}) : prepare_tile(d_k, KN, false, GK{});
-      mloc_sf = pv_tile(std::true_type{}, stat_t{}, VS * TILE, &tl_second, K_FIRST ? true : has_kn, s_b);
+      mloc_sf = pv_tile(std::true_type{}, stat_t{}, VS * TILE, &tl_second, K_FIRST ? true : has_kn, s_b, PAR,
+                        std::integral_constant<bool, SPLIT_SM>{});
     } else {
-      mloc_sf = pv_tile(std::true_type{}, stat_t{}, 0, nullptr, false, s_b);
+      mloc_sf = pv_tile(std::true_type{}, stat_t{}, 0, nullptr, false, s_b, PAR, std::false_type{});
     }
     if constexpr (!LAZY_MAX) maybe_rescale(mloc_sf);
   };
@@ -646,10 +689,11 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     else if (head_pending == 1) wait_vmcnt<LPT>();
     else wait_vmcnt<0>();
     __syncthreads();
-    qk_tile(std::false_type{}, std::false_type{}, 0, 0, s_e, s_e, nullptr, false);
+    qk_tile(std::false_type{}, std::false_type{}, 0, 0, s_e, s_e, 0, nullptr, false);
     if constexpr (MODE == KV_TOKENS) mask_tile(idw[0], idh[0], s_e);
     else mask_tile(hd[0], 0, s_e);
     maybe_rescale(row_stats(s_e));
+    if constexpr (SPLIT_SM) softmax_half(s_e, 0, 0);   // nothing to hide these under
 
     int it = 0;
     if constexpr (MODE != KV_TOKENS) {
@@ -681,7 +725,17 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
       }
     }
     // tail: softmax and P V of the last tile
-    if (it & 1) { softmax_only(s_o); softmax_close(s_o); } else { softmax_only(s_e); softmax_close(s_e); }
+    if (it & 1) {
+      if constexpr (SPLIT_SM) softmax_half(s_o, 1, 1); else softmax_only(s_o, 1);
+      softmax_close(s_o, 1);
+      if constexpr (SPLIT_SM) {
+#pragma unroll
+        for (int ks = 0; ks < 2 * NMB; ++ks) pb[0][ks] = pb[1][ks];
+      }
+    } else {
+      if constexpr (SPLIT_SM) softmax_half(s_e, 0, 1); else softmax_only(s_e, 0);
+      softmax_close(s_e, 0);
+    }
     wait_vmcnt<0>();
     if constexpr (MODE == KV_TOKENS) {
       // the id registers stay allocated until every id load has landed
@@ -691,7 +745,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     if constexpr (HAS_V) {
       __syncthreads();
       v_addr_refresh();
-      pv_tile(std::false_type{}, std::false_type{}, (uint32_t)(it & 1) * TILE, nullptr, false, s_e);
+      pv_tile(std::false_type{}, std::false_type{}, (uint32_t)(it & 1) * TILE, nullptr, false, s_e, 0, std::false_type{});
     }
   }
   __syncthreads();   // every wave is done with the ring
