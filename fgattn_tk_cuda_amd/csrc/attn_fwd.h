@@ -284,14 +284,13 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   using G1 = std::integral_constant<int, 1>;
   using G2 = std::integral_constant<int, 2>;
   if (ntiles > 0) issue_tile(head_desc(0), kslot(0), false, G0{});
-  // The Q loads are the only compiler-visible vector loads of the kernel.  They go out
-  // between the first copies so that their latency overlaps that of tile 0, and must have
-  // retired before the first counted wait.
+  // The Q loads go out behind the copy of K0 and are counted by hand like the copies (a load
+  // the compiler sees makes it wait for every copy issued before the first use of Q): the wait
+  // for K0 covers them.  Rows past the end of the sequence read the last row and are zeroed.
   u32x4 qf[NT];
-#pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    const u32x4 z = {0, 0, 0, 0};
-    qf[t] = qrow_ok ? *reinterpret_cast<const u32x4*>(qh + (size_t)qrow * D + 16 * t + 8 * g) : z;
+  {
+    const uint16_t* qsrc = qh + (size_t)(qrow_ok ? qrow : p.S - 1) * D + 8 * g;
+    load_q_uncounted<0, NT>(qf, qsrc);
   }
   int head_pending = 0;   // tile copies behind K0 when the first phase waits
   if (ntiles > 0) {
@@ -299,8 +298,6 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     if constexpr (HAS_V) { issue_tile(head_desc(0), vslot(0), true, G0{}); ++head_pending; }
     if (NK == 3 && 2 < ntiles) { issue_tile(head_desc(2), kslot(2), false, G2{}); ++head_pending; }
   }
-#pragma unroll
-  for (int t = 0; t < NT; ++t) asm volatile("" ::"v"(qf[t]));
 
   // Softmax state of this lane's query row.  Exponents are taken against a reference
   // mr_sf (in log2 units, = raw max * sf at the time it was set) that is only moved when
@@ -688,6 +685,11 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     else if (head_pending == 2) wait_vmcnt<2 * LPT>();
     else if (head_pending == 1) wait_vmcnt<LPT>();
     else wait_vmcnt<0>();
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      asm volatile("" : "+v"(qf[t]));
+      if (!qrow_ok) qf[t] = u32x4{0, 0, 0, 0};
+    }
     __syncthreads();
     qk_tile(std::false_type{}, std::false_type{}, 0, 0, s_e, s_e, 0, nullptr, false);
     if constexpr (MODE == KV_TOKENS) mask_tile(idw[0], idh[0], s_e);
@@ -747,6 +749,11 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
       v_addr_refresh();
       pv_tile(std::false_type{}, std::false_type{}, (uint32_t)(it & 1) * TILE, nullptr, false, s_e, 0, std::false_type{});
     }
+  } else {
+    // the Q loads still own their registers
+    wait_vmcnt<0>();
+#pragma unroll
+    for (int t = 0; t < NT; ++t) asm volatile("" ::"v"(qf[t]));
   }
   __syncthreads();   // every wave is done with the ring
 

@@ -106,6 +106,21 @@ __device__ __forceinline__ void dma16(const void* sbase, uint32_t voff, uint32_t
   const uint64_t sb = ((uint64_t)hi << 32) | lo;
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(voff), "s"(sb) : "memory");
 }
+// 16-byte global load that the compiler does not count either: the destination is valid only
+// behind a hand-placed vmcnt wait, after which the caller ties the registers to that point with
+// an empty asm ("+v") before their first use.
+template <int OFF>
+__device__ __forceinline__ void load16_uncounted(u32x4& dst, const void* ptr) {
+  asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=v"(dst) : "v"(ptr), "n"(OFF) : "memory");
+}
+// Q operands of the score product, k-steps T .. NT-1: 16 bytes every 32 from src.
+template <int T, int NT>
+__device__ __forceinline__ void load_q_uncounted(u32x4 (&qf)[NT], const void* src) {
+  if constexpr (T < NT) {
+    load16_uncounted<32 * T>(qf[T], src);
+    load_q_uncounted<T + 1, NT>(qf, src);
+  }
+}
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
