@@ -313,7 +313,13 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   constexpr float kTrigger = 256.f;   // 2^kSlack
   constexpr bool LAZY_MAX = !STATS;
   float mr_sf = kNegInf;
-  float base_eff = 0.f;    // mr_sf, or 0 while no key has been seen
+  // What the exponentials subtract: mr_sf once a key has been seen.  Before that, 0 where the
+  // row maxima are taken on every tile (every key so far was masked, p = exp2(-inf) = 0), but
+  // -inf with LAZY_MAX: a tile with a key then gives p = inf (NaN for its masked keys), the
+  // tile's sum trips the check below and the row gets its reference from that tile's true
+  // maximum, instead of keys being accumulated against a reference that was never recorded.
+  constexpr float kNoRef = LAZY_MAX ? kNegInf : 0.f;
+  float base_eff = kNoRef;
   float m_true = kNegInf;
   float l_run = 0.f;       // running denominator, this lane's keys only
   float l_tile = 0.f;      // sum of p over the tile whose softmax is in progress
@@ -423,7 +429,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
       const float new_sf = fmaxf(mr_sf, mloc_sf);
       const float alpha = (new_sf == kNegInf) ? 1.f : __builtin_amdgcn_exp2f(mr_sf - new_sf);
       mr_sf = new_sf;
-      base_eff = (new_sf == kNegInf) ? 0.f : new_sf;
+      base_eff = (new_sf == kNegInf) ? kNoRef : new_sf;
       l_run *= alpha;
       if constexpr (HAS_V) {
 #pragma unroll
@@ -459,9 +465,9 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
           if (half == 2 || (ks & 1) == half) asm volatile("" : "+v"(pb[SPLIT_SM ? par : 0][ks][i]));
     }
   };
-  auto softmax_only = [&](const f32x16 (&s)[NMB], int par) {
+  auto softmax_only = [&](const f32x16 (&s)[NMB], int par, float base) {
 #pragma unroll
-    for (int mb = 0; mb < NMB; ++mb) softmax_chunk(s, base_eff, mb, 0, 16, par);
+    for (int mb = 0; mb < NMB; ++mb) softmax_chunk(s, base, mb, 0, 16, par);
   };
   auto softmax_half = [&](const f32x16 (&s)[NMB], int par, int half) {
 #pragma unroll
@@ -473,7 +479,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     if constexpr (LAZY_MAX) {
       if (__any(!(l_tile <= kTrigger))) {
         maybe_rescale(row_stats(s));
-        softmax_only(s, par);
+        // a row that still has no reference has seen masked keys only: p = exp2(-inf - 0) = 0
+        softmax_only(s, par, mr_sf == kNegInf ? 0.f : mr_sf);
       }
     }
     l_run += l_tile;
@@ -728,14 +735,14 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     }
     // tail: softmax and P V of the last tile
     if (it & 1) {
-      if constexpr (SPLIT_SM) softmax_half(s_o, 1, 1); else softmax_only(s_o, 1);
+      if constexpr (SPLIT_SM) softmax_half(s_o, 1, 1); else softmax_only(s_o, 1, base_eff);
       softmax_close(s_o, 1);
       if constexpr (SPLIT_SM) {
 #pragma unroll
         for (int ks = 0; ks < 2 * NMB; ++ks) pb[0][ks] = pb[1][ks];
       }
     } else {
-      if constexpr (SPLIT_SM) softmax_half(s_e, 0, 1); else softmax_only(s_e, 0);
+      if constexpr (SPLIT_SM) softmax_half(s_e, 0, 1); else softmax_only(s_e, 0, base_eff);
       softmax_close(s_e, 0);
     }
     wait_vmcnt<0>();

@@ -207,6 +207,42 @@ def test_sp_attn_scores_that_outgrow_the_running_maximum(dev, D, qblk, growth):
 
 
 @pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("qblk", [64, 128])
+def test_sp_attn_first_tiles_without_a_key(dev, D, qblk):
+    """Lists that open with entries naming no key (ids beyond the sequence, or beyond a short kv
+    length): the row gets its exponent reference from the first tile that has a key, and the keys
+    of that tile and of every later one count."""
+    print("case sp_attn keyless first tiles", D, qblk, flush=True)
+    B, H, S = 1, 2, 512
+    rng = np.random.default_rng(41)
+    q, k, v = wl.randn_qkv(B, H, S, D, seed=40)
+    nq = orc.ceil_div(S, qblk)
+    ms = orc.padded_len(S)
+    idx = np.full((B, H, nq, ms), ms, np.int32)
+    num = np.zeros((B, H, nq), np.int32)
+    for h in range(H):
+        for i in range(nq):
+            dead = 32 * int(rng.integers(1, 7))            # 32 .. 192 leading entries without a key
+            live = int(rng.integers(1, 200))
+            idx[0, h, i, :dead] = S + rng.integers(0, 100, size=dead)
+            idx[0, h, i, dead:dead + live] = rng.integers(0, S, size=live)
+            num[0, h, i] = dead + live
+    o, lse = _run_tokens(dev, q, k, v, torch.from_numpy(idx), torch.from_numpy(num), qblk)
+    wo, wlse = orc.sp_attn(f32(q), f32(k), f32(v), idx, num, qblk=qblk)
+    assert_close_o(o, wo, "keyless first tiles, O")
+    assert_close_stat(lse, wlse, "keyless first tiles, lse", atol=1e-3)
+    # the same through a short kv length: most entries of a random list name no key
+    idx2 = np.full((B, H, nq, ms), ms, np.int32)
+    num2 = np.full((B, H, nq), 300, np.int32)
+    idx2[..., :300] = rng.integers(0, S, size=(B, H, nq, 300))
+    for kv_len in (39, 64, 65):
+        o2, lse2 = _run_tokens(dev, q, k, v, torch.from_numpy(idx2), torch.from_numpy(num2), qblk, kv_len=kv_len)
+        w2, wl2 = orc.sp_attn(f32(q), f32(k), f32(v), np.where(idx2 < kv_len, idx2, ms), num2, qblk=qblk)
+        assert_close_o(o2, w2, "kv_len %d, O" % kv_len)
+        assert_close_stat(lse2, wl2, "kv_len %d, lse" % kv_len, atol=1e-3)
+
+
+@pytest.mark.parametrize("D", [64, 128])
 @pytest.mark.parametrize("S,kv_len", [(512, 0), (1000, 0), (1000, 900), (130, 0)])
 def test_full_attn_and_stats(dev, D, S, kv_len):
     print("case full_attn", D, S, kv_len, flush=True)
