@@ -334,17 +334,21 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   // of the tile after, so that every multiply has the same vector-ALU work next to it (all of
   // it under QK^T leaves the vector ALU the bottleneck there and idle under P V).  Needs the
   // reference fixed before the tile's scores exist, which LAZY_MAX gives.
-  // (at d=128 a wave of a 128-row q-block has no registers left for the second set of operands)
-  constexpr bool SPLIT_SM = LAZY_MAX && HAS_V && (D == 64 || QBLK == 64);
+  constexpr bool SPLIT_SM = LAZY_MAX && HAS_V;
   u32x4 pb[SPLIT_SM ? 2 : 1][HAS_V ? 2 * NMB : 1];   // P^T operands, k-step 2mb + h; SPLIT_SM: by tile parity
 
   // Per-lane LDS addresses inside slot 0; slot, score block and k-step offsets are added
   // as constants (instruction immediates in the unrolled loop).
-  lds_cptr k_lo[NT];       // A operand of QK^T, k-step t, score block 0
+  // A operand of QK^T, k-step t, score block 0.  K_XOR (d=128 with 128-row q-blocks, where the
+  // registers do not reach and two Q operands were reloaded from scratch on every tile, each
+  // reload waiting for every tile copy in flight): only the address of k-step 0 is kept, that
+  // of k-step t is the same with t XORed into chunk bits 1-3.
+  constexpr bool K_XOR = (D == 128 && QBLK == 128);
+  lds_cptr k_lo[K_XOR ? 1 : NT];
   {
     const int krow = ksub * KW + ln;
 #pragma unroll
-    for (int t = 0; t < NT; ++t) k_lo[t] = smem_l + krow * ROWB + (((2 * t + g) ^ swz(krow)) << 4);
+    for (int t = 0; t < (K_XOR ? 1 : NT); ++t) k_lo[t] = smem_l + krow * ROWB + (((2 * t + g) ^ swz(krow)) << 4);
   }
   // Transposing V read: in each 16-lane group, lane i addresses 4 dims of key (i>>2);
   // lane j receives dim j of those 4 keys.  Keys 4g..4g+3 (+8 for the second read) of
@@ -365,9 +369,14 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   }
   // Called once per tile: hides v_base from loop-invariant code motion.
   // With a 64-row q-block there are registers to spare and the compiler may keep all of them.
+  uint32_t k_cur = 0;
   auto v_addr_refresh = [&]() {
     v_cur = v_base;
     if constexpr (QBLK != 64) asm volatile("" : "+v"(v_cur));
+    if constexpr (K_XOR) {
+      k_cur = (uint32_t)(uintptr_t)k_lo[0];
+      asm volatile("" : "+v"(k_cur));
+    }
   };
 
   // ---- building blocks --------------------------------------------------------------
@@ -486,21 +495,25 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     l_run += l_tile;
   };
 
-  // V^T operands of one 16-key step (PV group gi = 2mb + h), double-buffered over groups.
+  // V^T operands of one 16-key step (PV group gi = 2mb + h), double-buffered over groups; where
+  // the registers do not reach (K_XOR) one buffer, the operand of block db refilled for the
+  // next group as soon as its multiply of this group has been issued.
   constexpr int NG = 2 * NMB;
-  u32x2 va[HAS_V ? 2 : 1][HAS_V ? NDB : 1][2];
-  auto v_reads = [&](uint32_t vofs, int gi) {
+  constexpr int VB = K_XOR ? 1 : 2;
+  u32x2 va[HAS_V ? VB : 1][HAS_V ? NDB : 1][2];
+  auto v_read_db = [&](uint32_t vofs, int gi, int db) {
     if constexpr (HAS_V) {
-#pragma unroll
-      for (int db = 0; db < NDB; ++db) {
-        const uint32_t x1 = v_cur ^ (uint32_t)(db << 6);
-        const uint32_t x2 = x1 ^ 32u;
-        const lds_cptr a1 = (lds_cptr)(uintptr_t)x1 + vofs + gi * 16 * ROWB;
-        const lds_cptr a2 = (lds_cptr)(uintptr_t)x2 + vofs + gi * 16 * ROWB + 8 * ROWB;
-        va[gi & 1][db][0] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((SPATTN_LDS s16x4*)a1));
-        va[gi & 1][db][1] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((SPATTN_LDS s16x4*)a2));
-      }
+      const uint32_t x1 = v_cur ^ (uint32_t)(db << 6);
+      const uint32_t x2 = x1 ^ 32u;
+      const lds_cptr a1 = (lds_cptr)(uintptr_t)x1 + vofs + gi * 16 * ROWB;
+      const lds_cptr a2 = (lds_cptr)(uintptr_t)x2 + vofs + gi * 16 * ROWB + 8 * ROWB;
+      va[gi % VB][db][0] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((SPATTN_LDS s16x4*)a1));
+      va[gi % VB][db][1] = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((SPATTN_LDS s16x4*)a2));
     }
+  };
+  auto v_reads = [&](uint32_t vofs, int gi) {
+#pragma unroll
+    for (int db = 0; db < (HAS_V ? NDB : 0); ++db) v_read_db(vofs, gi, db);
   };
 
   // s_out^T = K Q^T from the K tile at ring offset kofs (bytes), one 32-key block at a
@@ -522,7 +535,14 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
       u32x4 ka[NT];
       auto k_reads = [&](int t0, int t1) {
 #pragma unroll
-        for (int t = t0; t < t1; ++t) ka[t] = *(SPATTN_LDS const u32x4*)(k_lo[t] + kofs + mb * 32 * ROWB);
+        for (int t = t0; t < t1; ++t) {
+          if constexpr (K_XOR) {
+            const uint32_t a0 = k_cur ^ (uint32_t)(t << 5);
+            ka[t] = *(SPATTN_LDS const u32x4*)((lds_cptr)(uintptr_t)a0 + kofs + mb * 32 * ROWB);
+          } else {
+            ka[t] = *(SPATTN_LDS const u32x4*)(k_lo[t] + kofs + mb * 32 * ROWB);
+          }
+        }
         __builtin_amdgcn_sched_barrier(0);
       };
       // the operands arrive in two batches, to bound the registers they hold
@@ -586,12 +606,13 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
       if constexpr (!decltype(first_loaded)::value) v_reads(vofs, 0);
 #pragma unroll
       for (int gi = 0; gi < NG; ++gi) {
-        if (gi + 1 < NG) v_reads(vofs, gi + 1);
+        if (VB == 2 && gi + 1 < NG) v_reads(vofs, gi + 1);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int db = 0; db < NDB; ++db) {
-          const u32x4 a = {va[gi & 1][db][0][0], va[gi & 1][db][0][1], va[gi & 1][db][1][0], va[gi & 1][db][1][1]};
+          const u32x4 a = {va[gi % VB][db][0][0], va[gi % VB][db][0][1], va[gi % VB][db][1][0], va[gi % VB][db][1][1]};
           oacc[db] = mfma32(a, pb[SPLIT_SM ? par : 0][gi], oacc[db]);
+          if (VB == 1 && gi + 1 < NG) v_read_db(vofs, gi + 1, db);
           const int m = gi * NDB + db;
           if constexpr (EARLY_SM) {
             if (m % MPP == 0) softmax_chunk(s_next, base, (m / MPP) / 4, 2 * ((m / MPP) % 4), 2, par ^ 1);
@@ -698,6 +719,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
       if (!qrow_ok) qf[t] = u32x4{0, 0, 0, 0};
     }
     __syncthreads();
+    v_addr_refresh();
     qk_tile(std::false_type{}, std::false_type{}, 0, 0, s_e, s_e, 0, nullptr, false);
     if constexpr (MODE == KV_TOKENS) mask_tile(idw[0], idh[0], s_e);
     else mask_tile(hd[0], 0, s_e);
