@@ -124,3 +124,38 @@ def test_block_lists_random(dev, seed):
     wo, wlse = orc.sp_attn(f32(q), f32(k), f32(v), tok, num, qblk=qblk)
     assert_close_o(f32(o), wo, "random block lists, O")
     assert_close_stat(f32(lse), wlse, "random block lists, lse", atol=2e-3)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_operator_sp_attn_equals_the_c_abi_bit_for_bit(dev, seed):
+    """torch.ops.cuda_attn.sp_attn (which orders the q-blocks by list length and launches the
+    ordered entry point) against the plain C-ABI launch on the same ragged lists."""
+    import fgattn_tk_cuda_amd.spattn.cuda_attn  # noqa: F401
+    rng = np.random.default_rng(7000 + seed)
+    B, H = int(rng.integers(1, 3)), int(rng.integers(1, 4))
+    S = int(rng.choice([192, 449, 700, 1024]))
+    D = int(rng.choice([64, 128]))
+    qblk = int(rng.choice([64, 128]))
+    print("case op vs C ABI", seed, B, H, S, D, qblk, flush=True)
+    q, k, v = wl.randn_qkv(B, H, S, D, seed=200 + seed)
+    nq = orc.ceil_div(S, qblk)
+    ms = orc.padded_len(S)
+    idx = np.full((B, H, nq, ms), ms, np.int32)
+    num = np.zeros((B, H, nq), np.int32)
+    for b in range(B):
+        for h in range(H):
+            for i in range(nq):
+                # list lengths spread over more than a factor of two, so that the order is not the default one
+                c = int(rng.choice([0, 1, 17, 64, 200, S])) if rng.random() < 0.5 else int(rng.integers(1, S + 1))
+                c = min(c, ms)
+                idx[b, h, i, :c] = rng.integers(0, S, size=c)
+                num[b, h, i] = c
+    qd, kd, vd, idxd, numd = to_dev(dev, q, k, v, torch.from_numpy(idx), torch.from_numpy(num))
+    o_op = torch.full_like(qd, float("nan"))
+    torch.ops.cuda_attn.sp_attn(o_op, qd, kd, vd, idxd, numd)
+    o_c = torch.full_like(qd, float("nan"))
+    capi.sp_attn(o_c, qd, kd, vd, idxd, numd, qblk=qblk)
+    torch.cuda.synchronize()
+    assert torch.equal(o_op.view(torch.int16), o_c.view(torch.int16))
+    wo, _ = orc.sp_attn(f32(q), f32(k), f32(v), idx, num, qblk=qblk)
+    assert_close_o(f32(o_op), wo, "operator sp_attn vs oracle")
