@@ -26,7 +26,7 @@ HIP_SOURCES = [
     "attn_inst_blocks.hip",
     "attn_inst_dense.hip",
     "mask_kernels.hip",
-    "bitmask_kernels.hip", "topk_kernels.hip", "order_kernels.hip",
+    "bitmask_kernels.hip", "blocklist_kernels.hip", "topk_kernels.hip", "order_kernels.hip",
     "capi.hip",
 ]
 

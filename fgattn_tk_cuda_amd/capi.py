@@ -38,6 +38,9 @@ _SIGNATURES = {
     "spattn_maxq_denom": (_c_int, [_c_void_p] * 4 + [_c_int] * 5 + [_c_float, _c_void_p]),
     "spattn_booleanmask_128": (_c_int, [_c_void_p, _c_float, _c_int] + [_c_void_p] * 4 + [_c_int] * 5 + [_c_float, _c_void_p]),
     "spattn_booleanmask_to_indexmask": (_c_int, [_c_void_p] * 3 + [_c_int] * 5 + [_c_void_p]),
+    "spattn_booleanmask_packed": (_c_int, [_c_void_p, _c_float, _c_int, _c_int] + [_c_void_p] * 4 + [_c_int] * 5 + [_c_float, _c_void_p]),
+    "spattn_packedmask_to_blocklists": (_c_int, [_c_void_p] * 4 + [_c_int] * 6 + [_c_void_p]),
+    "spattn_booleanmask_to_blocklists": (_c_int, [_c_void_p] * 4 + [_c_int] * 6 + [_c_void_p]),
     "spattn_pack_mask": (_c_int, [_c_void_p] * 2 + [_c_int] * 4 + [_c_void_p]),
     "spattn_packedmask_to_indexmask": (_c_int, [_c_void_p] * 3 + [_c_int] * 5 + [_c_void_p]),
     "spattn_qk_topkmask_indices": (_c_int, [_c_void_p] * 6 + [_c_int] * 9 + [_c_void_p]),
@@ -207,6 +210,50 @@ def booleanmask_to_indexmask(kv_indices, kv_num_indices, booleanmask, seq, *, st
         raise ValueError("kv_indices / kv_num_indices do not match booleanmask")
     _check(load().spattn_booleanmask_to_indexmask(_ptr(kv_indices, i32), _ptr(kv_num_indices, i32),
                                                   _ptr(booleanmask, i32), B, H, int(seq), SB, MS, _stream(stream)))
+
+
+def booleanmask_packed(packed, max_q, denom, q, k, threshold, *, qblk=128, kv_len=0, scale=0.0, stream=None):
+    """Threshold sweep with a bit-packed result: packed uint8 [B,H,ceil(S/qblk),mask_stride/8], bit
+    (c & 7) of byte c >> 3 set where some row of the q-block has softmax(row, c) > threshold."""
+    B, H, S, D = _bhsd(q)
+    _need_padded(max_q, denom, B, H, S)
+    if qblk not in (64, 128):
+        raise ValueError("qblk must be 64 or 128")
+    if packed.dim() != 4 or tuple(packed.shape[:3]) != (B, H, (S + qblk - 1) // qblk):
+        raise ValueError("packed must be uint8 [B,H,ceil(S/qblk),mask_stride/8]")
+    _check(load().spattn_booleanmask_packed(_ptr(packed, torch.uint8), float(threshold), int(packed.shape[3]) * 8,
+                                            int(qblk), _ptr(max_q, f32), _ptr(denom, f32), _ptr(q, bf16), _ptr(k, bf16),
+                                            B, H, S, D, kv_len, scale, _stream(stream)))
+
+
+def _blocklist_args(blk_indices, blk_counts, blockmask, B, H, SB, MS):
+    if blk_indices.dim() != 4 or tuple(blk_indices.shape[:3]) != (B, H, SB) or blk_counts.numel() != B * H * SB:
+        raise ValueError("blk_indices must be [B,H,SB,max_blocks] and blk_counts hold B*H*SB entries")
+    if blockmask is not None and tuple(blockmask.shape) != (B, H, SB, MS // 64):
+        raise ValueError("blockmask must be uint8 [B,H,SB,mask_stride/64]")
+
+
+def packedmask_to_blocklists(blk_indices, blk_counts, packed, seq, *, blockmask=None, stream=None):
+    """Ascending lists of the 64-key blocks that hold a set key c < seq, from a bit-packed mask
+    (uint8 [B,H,SB,mask_stride/8]); blockmask: optional uint8 [B,H,SB,mask_stride/64] output."""
+    if packed.dim() != 4:
+        raise ValueError("packed must be [B,H,SB,mask_stride/8]")
+    B, H, SB, MB = (int(x) for x in packed.shape)
+    _blocklist_args(blk_indices, blk_counts, blockmask, B, H, SB, MB * 8)
+    _check(load().spattn_packedmask_to_blocklists(_ptr(blk_indices, i32), _ptr(blk_counts, i32),
+                                                  _ptr(blockmask, torch.uint8), _ptr(packed, torch.uint8), B, H,
+                                                  int(seq), SB, MB * 8, int(blk_indices.shape[3]), _stream(stream)))
+
+
+def booleanmask_to_blocklists(blk_indices, blk_counts, booleanmask, seq, *, blockmask=None, stream=None):
+    """The same from the int32 vote mask [B,H,SB,mask_stride]."""
+    if booleanmask.dim() != 4:
+        raise ValueError("booleanmask must be [B,H,SB,mask_stride]")
+    B, H, SB, MS = (int(x) for x in booleanmask.shape)
+    _blocklist_args(blk_indices, blk_counts, blockmask, B, H, SB, MS)
+    _check(load().spattn_booleanmask_to_blocklists(_ptr(blk_indices, i32), _ptr(blk_counts, i32),
+                                                   _ptr(blockmask, torch.uint8), _ptr(booleanmask, i32), B, H, int(seq),
+                                                   SB, MS, int(blk_indices.shape[3]), _stream(stream)))
 
 
 def pack_mask(packed, booleanmask, *, stream=None):

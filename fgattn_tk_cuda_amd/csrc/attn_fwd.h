@@ -97,6 +97,9 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   // a caller-given work order (longest lists first) replaces the XCD-contiguous default
   const int wg = p.order ? ((const __attribute__((address_space(4))) int*)p.order)[blockIdx.x]
                          : xcd_remap(blockIdx.x, total);
+  // an entry of a work order that names no q-block: nothing is addressed (wave-uniform, ahead
+  // of every copy and barrier)
+  if ((unsigned)wg >= (unsigned)total) return;
   const int qb = wg % p.nqblk;
   const int bh = wg / p.nqblk;
 

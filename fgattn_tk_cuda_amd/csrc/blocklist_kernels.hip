@@ -1,0 +1,126 @@
+// Key mask -> KV-block mask -> KV-block index lists, for gfx950.
+//
+// The reference's pre-pass ends in per-key lists (include/mask_utils.cuh:273-302).  The block
+// form of the same step: key block J (64 keys) of a mask row is kept when any of its keys
+// c < kv_len is set,
+//   MB[row, J] = OR_{c in 64J .. 64J+63, c < kv_len} M[row, c],
+// and the kept block ids of a row are written in ascending order, followed by the caller's
+// fill, with the count next to them - what the block-list attention kernel walks.
+//
+// Two sources: the bit-packed mask (one 64-bit word is one block; 1/32 of the bytes) and the
+// reference's int32 vote mask (a pure HBM stream like the per-key compaction).  One wave owns
+// one row; a lane stands for one block of a group of 64, so the rank of a kept block is a
+// wave ballot and a bit count - no atomics, deterministic, ascending.
+#include "common.h"
+#include "dispatch.h"
+
+namespace spattn {
+
+constexpr int kBlockListMaxGrid = 2048;   // workgroups of 4 waves; further rows in further rounds
+
+// Appends the kept blocks of one group of 64 (lane = block J0 + lane) to the row's list.
+__device__ __forceinline__ void append_blocks(bool keep, int J, int nblk, int& count, int* __restrict__ dst,
+                                              unsigned char* __restrict__ mrow, int max_blocks) {
+  const unsigned long long b = __ballot(keep);
+  const int pos = count + __builtin_amdgcn_mbcnt_hi((unsigned)(b >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)b, 0));
+  if (keep && pos < max_blocks) dst[pos] = J;
+  if (mrow != nullptr && J < nblk) mrow[J] = keep ? 1 : 0;
+  count += __popcll(b);
+}
+
+__global__ __launch_bounds__(256) void packed_to_blocklists_kernel(int* __restrict__ blk_indices,
+                                                                   int* __restrict__ blk_counts,
+                                                                   unsigned char* __restrict__ blockmask,
+                                                                   const uint32_t* __restrict__ packed, int rows,
+                                                                   int mask_stride, int kv_len, int max_blocks) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int nblk = mask_stride >> 6;
+  const int lim = kv_len < mask_stride ? kv_len : mask_stride;
+  for (int row = blockIdx.x * 4 + wave; row < rows; row += gridDim.x * 4) {
+    const u32x2* __restrict__ src = reinterpret_cast<const u32x2*>(packed + (size_t)row * (mask_stride >> 5));
+    int* __restrict__ dst = blk_indices + (size_t)row * max_blocks;
+    unsigned char* mrow = blockmask ? blockmask + (size_t)row * nblk : nullptr;
+    int count = 0;
+    for (int J0 = 0; J0 < nblk; J0 += 64) {
+      const int J = J0 + lane;
+      u32x2 w = {0u, 0u};
+      if (J < nblk) w = src[J];
+      unsigned long long bits = ((unsigned long long)w[1] << 32) | w[0];
+      const int valid = lim - J * 64;   // keys of this block below the kv length
+      if (valid <= 0) bits = 0;
+      else if (valid < 64) bits &= (1ull << valid) - 1ull;
+      append_blocks(bits != 0, J, nblk, count, dst, mrow, max_blocks);
+    }
+    if (lane == 0) blk_counts[row] = count;
+  }
+}
+
+// int32 votes: a wave step covers 64 blocks = 4096 keys with 16 loads of 16 bytes per lane, all
+// requested before the first is looked at.  Load u of lane l holds keys 256u + 4l .. +3 of the
+// step, so block 4u + b of the step is lanes 16b .. 16b+15 of load u: one ballot per load, four
+// 16-bit fields per ballot.
+__global__ __launch_bounds__(256) void votes_to_blocklists_kernel(int* __restrict__ blk_indices,
+                                                                  int* __restrict__ blk_counts,
+                                                                  unsigned char* __restrict__ blockmask,
+                                                                  const int* __restrict__ votes, int rows,
+                                                                  int mask_stride, int kv_len, int max_blocks) {
+  constexpr int U = 16;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int nblk = mask_stride >> 6;
+  const int lim = kv_len < mask_stride ? kv_len : mask_stride;
+  for (int row = blockIdx.x * 4 + wave; row < rows; row += gridDim.x * 4) {
+    const int* __restrict__ src = votes + (size_t)row * mask_stride;
+    int* __restrict__ dst = blk_indices + (size_t)row * max_blocks;
+    unsigned char* mrow = blockmask ? blockmask + (size_t)row * nblk : nullptr;
+    int count = 0;
+    for (int J0 = 0; J0 < nblk; J0 += 64) {
+      const int e_base = J0 * 64 + 4 * lane;
+      i32x4 v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int e0 = e_base + u * 256;
+        const i32x4 z = {0, 0, 0, 0};
+        // mask_stride is a multiple of 4: a vector that starts inside the row stays inside it
+        v[u] = (e0 < lim) ? __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(src + e0)) : z;
+      }
+      unsigned long long word = 0;   // bit j: block J0 + j has a key
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int e0 = e_base + u * 256;
+        const bool f = (v[u][0] > 0 && e0 < lim) || (v[u][1] > 0 && e0 + 1 < lim) || (v[u][2] > 0 && e0 + 2 < lim) ||
+                       (v[u][3] > 0 && e0 + 3 < lim);
+        const unsigned long long b = __ballot(f);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if ((b >> (16 * j)) & 0xffffull) word |= 1ull << (4 * u + j);
+      }
+      append_blocks((word >> lane) & 1ull, J0 + lane, nblk, count, dst, mrow, max_blocks);
+    }
+    if (lane == 0) blk_counts[row] = count;
+  }
+}
+
+static int blocklist_grid(int rows) {
+  int grid = (rows + 3) / 4;
+  return grid > kBlockListMaxGrid ? kBlockListMaxGrid : grid;
+}
+
+hipError_t run_packed_to_blocklists(int* blk_indices, int* blk_counts, unsigned char* blockmask, const uint32_t* packed,
+                                    int rows, int mask_stride, int kv_len, int max_blocks, hipStream_t stream) {
+  if (rows <= 0) return hipSuccess;
+  hipLaunchKernelGGL(packed_to_blocklists_kernel, dim3(blocklist_grid(rows)), dim3(256), 0, stream, blk_indices,
+                     blk_counts, blockmask, packed, rows, mask_stride, kv_len, max_blocks);
+  return hipGetLastError();
+}
+
+hipError_t run_votes_to_blocklists(int* blk_indices, int* blk_counts, unsigned char* blockmask, const int* votes,
+                                   int rows, int mask_stride, int kv_len, int max_blocks, hipStream_t stream) {
+  if (rows <= 0) return hipSuccess;
+  hipLaunchKernelGGL(votes_to_blocklists_kernel, dim3(blocklist_grid(rows)), dim3(256), 0, stream, blk_indices,
+                     blk_counts, blockmask, votes, rows, mask_stride, kv_len, max_blocks);
+  return hipGetLastError();
+}
+
+}  // namespace spattn

@@ -20,7 +20,8 @@ inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s);
 int check_qkv(const void* q, const void* k, int B, int H, int S, int D) {
   if (!q || !k) return SPATTN_ERR_NULL;
   if (D != 64 && D != 128) return SPATTN_ERR_HEAD_DIM;
-  if (B <= 0 || H <= 0 || S <= 0) return SPATTN_ERR_SHAPE;
+  // tile descriptors carry a row number in 24 bits
+  if (B <= 0 || H <= 0 || S <= 0 || S >= (1 << 24)) return SPATTN_ERR_SHAPE;
   if (misaligned(q) || misaligned(k)) return SPATTN_ERR_ALIGN;
   return SPATTN_OK;
 }
@@ -128,9 +129,46 @@ int spattn_booleanmask_128(int* booleanmask, float threshold, int mask_stride, c
   if (mask_stride <= 0 || mask_stride % 128 != 0) return done(SPATTN_ERR_STRIDE);
   const int kv = (kv_len <= 0 || kv_len > S) ? S : kv_len;
   const float sc = scale > 0.f ? scale : 1.0f / sqrtf((float)D);
-  return from_hip(spattn::run_booleanmask(booleanmask, threshold, mask_stride, max_q, denom,
+  return from_hip(spattn::run_booleanmask(booleanmask, 0, threshold, mask_stride, max_q, denom,
                                           static_cast<const uint16_t*>(q), static_cast<const uint16_t*>(k), B, H, S, D,
                                           kv < mask_stride ? kv : mask_stride, sc, as_stream(stream)));
+}
+
+int spattn_booleanmask_packed(void* packed, float threshold, int mask_stride, int qblk, const float* max_q,
+                              const float* denom, const void* q, const void* k, int B, int H, int S, int D, int kv_len,
+                              float scale, void* stream) {
+  if (int st = check_qkv(q, k, B, H, S, D)) return done(st);
+  if (!packed || !max_q || !denom) return done(SPATTN_ERR_NULL);
+  if (qblk != 64 && qblk != 128) return done(SPATTN_ERR_QBLK);
+  if (mask_stride <= 0 || mask_stride % 128 != 0) return done(SPATTN_ERR_STRIDE);
+  if (misaligned(packed)) return done(SPATTN_ERR_ALIGN);
+  const int kv = (kv_len <= 0 || kv_len > S) ? S : kv_len;
+  const float sc = scale > 0.f ? scale : 1.0f / sqrtf((float)D);
+  return from_hip(spattn::run_booleanmask(packed, qblk, threshold, mask_stride, max_q, denom,
+                                          static_cast<const uint16_t*>(q), static_cast<const uint16_t*>(k), B, H, S, D,
+                                          kv < mask_stride ? kv : mask_stride, sc, as_stream(stream)));
+}
+
+int spattn_packedmask_to_blocklists(int* blk_indices, int* blk_counts, void* blockmask, const void* packed, int B, int H,
+                                    int seq, int seqblocks, int mask_stride, int max_blocks, void* stream) {
+  if (!blk_indices || !blk_counts || !packed) return done(SPATTN_ERR_NULL);
+  if (B <= 0 || H <= 0 || seqblocks <= 0 || seq < 0 || max_blocks <= 0) return done(SPATTN_ERR_SHAPE);
+  if (mask_stride <= 0 || mask_stride % 128 != 0) return done(SPATTN_ERR_STRIDE);
+  if (misaligned(packed)) return done(SPATTN_ERR_ALIGN);
+  return from_hip(spattn::run_packed_to_blocklists(blk_indices, blk_counts, static_cast<unsigned char*>(blockmask),
+                                                   static_cast<const uint32_t*>(packed), B * H * seqblocks, mask_stride,
+                                                   seq, max_blocks, as_stream(stream)));
+}
+
+int spattn_booleanmask_to_blocklists(int* blk_indices, int* blk_counts, void* blockmask, const int* booleanmask, int B,
+                                     int H, int seq, int seqblocks, int mask_stride, int max_blocks, void* stream) {
+  if (!blk_indices || !blk_counts || !booleanmask) return done(SPATTN_ERR_NULL);
+  if (B <= 0 || H <= 0 || seqblocks <= 0 || seq < 0 || max_blocks <= 0) return done(SPATTN_ERR_SHAPE);
+  if (mask_stride <= 0 || mask_stride % 128 != 0) return done(SPATTN_ERR_STRIDE);
+  if (misaligned(booleanmask)) return done(SPATTN_ERR_ALIGN);
+  return from_hip(spattn::run_votes_to_blocklists(blk_indices, blk_counts, static_cast<unsigned char*>(blockmask),
+                                                  booleanmask, B * H * seqblocks, mask_stride, seq, max_blocks,
+                                                  as_stream(stream)));
 }
 
 int spattn_booleanmask_to_indexmask(int* kv_indices, int* num_kv_indices, const int* booleanmask, int B, int H, int seq,
@@ -272,6 +310,6 @@ const char* spattn_status_string(int status) {
   }
 }
 
-int spattn_version(void) { return 1; }
+int spattn_version(void) { return 2; }
 
 }  // extern "C"

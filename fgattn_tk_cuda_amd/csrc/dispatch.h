@@ -10,9 +10,9 @@ hipError_t run_attn_blocks(const AttnParams& p, int D, int qblk, hipStream_t str
 hipError_t run_attn_dense(const AttnParams& p, int D, bool has_v, bool stats, hipStream_t stream);
 
 // mask_kernels.hip
-hipError_t run_booleanmask(int* mask, float thresh, int mask_stride, const float* max_q, const float* denom,
-                           const uint16_t* q, const uint16_t* k, int B, int H, int S, int D, int kv_len, float scale,
-                           hipStream_t stream);
+hipError_t run_booleanmask(void* out, int out_rows, float thresh, int mask_stride, const float* max_q,
+                           const float* denom, const uint16_t* q, const uint16_t* k, int B, int H, int S, int D,
+                           int kv_len, float scale, hipStream_t stream);
 hipError_t run_compact(int* kv_indices, int* kv_num, const int* mask, int rows, int mask_stride, int kv_len,
                        hipStream_t stream);
 hipError_t run_all_index(int* kv_indices, int* kv_num, int rows, int mask_stride, int seq, hipStream_t stream);
@@ -21,6 +21,12 @@ hipError_t run_all_index(int* kv_indices, int* kv_num, int rows, int mask_stride
 hipError_t run_pack_mask(uint32_t* packed, const int* mask, int rows, int mask_stride, hipStream_t stream);
 hipError_t run_packed_to_indexmask(int* kv_indices, int* kv_num, const uint32_t* packed, int rows, int mask_stride,
                                    int kv_len, hipStream_t stream);
+
+// blocklist_kernels.hip
+hipError_t run_packed_to_blocklists(int* blk_indices, int* blk_counts, unsigned char* blockmask, const uint32_t* packed,
+                                    int rows, int mask_stride, int kv_len, int max_blocks, hipStream_t stream);
+hipError_t run_votes_to_blocklists(int* blk_indices, int* blk_counts, unsigned char* blockmask, const int* votes,
+                                   int rows, int mask_stride, int kv_len, int max_blocks, hipStream_t stream);
 
 // topk_kernels.hip
 hipError_t run_topk_mask(int* kv_indices, int* kv_num, uint16_t* score, uint16_t* qmean, const uint16_t* q,

@@ -31,8 +31,18 @@ namespace spattn {
 // subtraction, the vector ALU only takes the maximum of the 8 registers a lane holds of a
 // 16-row group (v_max3) and compares it with 0; one exchange with lane n^32 finishes the 8
 // votes of a key.  The vote count is stored, not accumulated.
+//
+// Three output forms (OUT), the sweep is the same:
+//   OUT_VOTES   int32 vote count per (128-row q-block, key)         - the reference's mask
+//   OUT_BITS128 one bit per (128-row q-block, key): count > 0, 32 keys per stored word,
+//               least significant bit first - 1/32 of the bytes, the layout of the mask cache
+//   OUT_BITS64  one bit per (64-row q-block, key): the four 16-row groups of each half of the
+//               128-row block vote separately; rows 2I and 2I+1 of the output
+// A wave holds the votes of 32 consecutive keys in 32 lanes, so a word is one ballot.
 // ------------------------------------------------------------------------------------
-template <int D>
+enum MaskOut : int { OUT_VOTES = 0, OUT_BITS128 = 1, OUT_BITS64 = 2 };
+
+template <int D, int OUT>
 __global__ __launch_bounds__(256, 2) void booleanmask_kernel(int* __restrict__ mask, const float* __restrict__ max_q,
                                                               const float* __restrict__ denom,
                                                               const uint16_t* __restrict__ q,
@@ -106,6 +116,17 @@ __global__ __launch_bounds__(256, 2) void booleanmask_kernel(int* __restrict__ m
 
   int* mrow = mask + ((size_t)bh * SB + qb) * mask_stride;
   const int nkb = (mask_stride + 31) >> 5;
+  // bit outputs: rows of mask_stride / 32 words; with 64-row q-blocks the last 128-row block
+  // of a head may have one half only
+  const int nq64 = (S + 63) >> 6;
+  uint32_t* brow0 = nullptr;
+  uint32_t* brow1 = nullptr;
+  if constexpr (OUT == OUT_BITS128) {
+    brow0 = reinterpret_cast<uint32_t*>(mask) + ((size_t)bh * SB + qb) * (size_t)nkb;
+  } else if constexpr (OUT == OUT_BITS64) {
+    brow0 = reinterpret_cast<uint32_t*>(mask) + ((size_t)bh * nq64 + 2 * qb) * (size_t)nkb;
+    if (2 * qb + 1 < nq64) brow1 = brow0 + nkb;
+  }
 
   // Ring layout: key row r of a block at r * 2D bytes, its 16-byte chunk c at c ^ kswz(r),
   // which spreads chunk 2t+g of the 32 rows a half wave reads over all bank groups.  Copy i
@@ -211,7 +232,24 @@ __global__ __launch_bounds__(256, 2) void booleanmask_kernel(int* __restrict__ m
     pair_values(__builtin_bit_cast(float, votes), lo_, hi_);   // v_permlane32_swap, no LDS
     votes = __builtin_bit_cast(unsigned, lo_) | __builtin_bit_cast(unsigned, hi_);
     const int key = kb * 32 + ln;   // negative for the block "before the first": nothing is stored
-    if (g == 0 && (unsigned)key < (unsigned)mask_stride) mrow[key] = (key < kv_len) ? __popc(votes) : 0;
+    if constexpr (OUT == OUT_VOTES) {
+      if (g == 0 && (unsigned)key < (unsigned)mask_stride) mrow[key] = (key < kv_len) ? __popc(votes) : 0;
+    } else {
+      // lanes n and n + 32 hold the same votes: the low word of a ballot is the 32 keys
+      const bool live = (unsigned)key < (unsigned)kv_len;
+      const bool store = lane == 0 && (unsigned)kb < (unsigned)nkb;
+      if constexpr (OUT == OUT_BITS128) {
+        const uint32_t w = (uint32_t)__ballot(live && votes != 0);
+        if (store) brow0[kb] = w;
+      } else {
+        const uint32_t w0 = (uint32_t)__ballot(live && (votes & 0x0fu) != 0);
+        const uint32_t w1 = (uint32_t)__ballot(live && (votes & 0xf0u) != 0);
+        if (store) {
+          brow0[kb] = w0;
+          if (brow1 != nullptr) brow1[kb] = w1;
+        }
+      }
+    }
   };
   // Half H: multiplies pair H&1 of block kb into acc[H % NACC] and reduces the accumulators
   // of the half before.
@@ -284,22 +322,39 @@ __global__ __launch_bounds__(256, 2) void booleanmask_kernel(int* __restrict__ m
   }
 }
 
-hipError_t run_booleanmask(int* mask, float thresh, int mask_stride, const float* max_q, const float* denom,
-                           const uint16_t* q, const uint16_t* k, int B, int H, int S, int D, int kv_len, float scale,
-                           hipStream_t stream) {
+template <int D, int OUT>
+static void launch_booleanmask(int* mask, float lt, int mask_stride, const float* max_q, const float* denom,
+                               const uint16_t* q, const uint16_t* k, int HB, int S, int kv_len, int Sp, int SB, float sf,
+                               hipStream_t stream) {
+  hipLaunchKernelGGL((booleanmask_kernel<D, OUT>), dim3(SB * HB, 1, 1), dim3(256), 0, stream, mask, max_q, denom, q, k,
+                     lt, mask_stride, HB, S, kv_len, Sp, SB, sf);
+}
+
+// out_rows: 0 = int32 vote counts; 128 / 64 = bit rows per q-block of that many query rows.
+hipError_t run_booleanmask(void* out, int out_rows, float thresh, int mask_stride, const float* max_q,
+                           const float* denom, const uint16_t* q, const uint16_t* k, int B, int H, int S, int D,
+                           int kv_len, float scale, hipStream_t stream) {
   const int SB = (S + 127) / 128;
   const int Sp = SB * 128;
   const float sf = kLog2e * scale;
   const float lt = thresh > 0.f ? log2f(thresh) : -__builtin_huge_valf();
   const int total = SB * H * B;
   if (total <= 0) return hipSuccess;
+  int* m = static_cast<int*>(out);
+  const int HB = H * B;
+#define SPATTN_MASK_CASE(DD, OO) launch_booleanmask<DD, OO>(m, lt, mask_stride, max_q, denom, q, k, HB, S, kv_len, Sp, SB, sf, stream)
   if (D == 128) {
-    hipLaunchKernelGGL(booleanmask_kernel<128>, dim3(total, 1, 1), dim3(256), 0, stream, mask, max_q, denom, q, k, lt,
-                       mask_stride, H * B, S, kv_len, Sp, SB, sf);
+    if (out_rows == 0) SPATTN_MASK_CASE(128, OUT_VOTES);
+    else if (out_rows == 128) SPATTN_MASK_CASE(128, OUT_BITS128);
+    else if (out_rows == 64) SPATTN_MASK_CASE(128, OUT_BITS64);
+    else return hipErrorInvalidValue;
   } else {
-    hipLaunchKernelGGL(booleanmask_kernel<64>, dim3(total, 1, 1), dim3(256), 0, stream, mask, max_q, denom, q, k, lt,
-                       mask_stride, H * B, S, kv_len, Sp, SB, sf);
+    if (out_rows == 0) SPATTN_MASK_CASE(64, OUT_VOTES);
+    else if (out_rows == 128) SPATTN_MASK_CASE(64, OUT_BITS128);
+    else if (out_rows == 64) SPATTN_MASK_CASE(64, OUT_BITS64);
+    else return hipErrorInvalidValue;
   }
+#undef SPATTN_MASK_CASE
   return hipGetLastError();
 }
 

@@ -28,7 +28,7 @@ extern "C" {
 #define SPATTN_ERR_STRIDE -3     /* mask_stride is not a positive multiple of 128 */
 #define SPATTN_ERR_QBLK -4       /* q-block is not 64 or 128 */
 #define SPATTN_ERR_ALIGN -5      /* a pointer is not 16-byte aligned */
-#define SPATTN_ERR_SHAPE -6      /* a size is not positive / inconsistent */
+#define SPATTN_ERR_SHAPE -6      /* a size is not positive / inconsistent, or seq >= 2^24 */
 
 /* ---- group 1: the reference's binding surface ------------------------------------ */
 
@@ -121,6 +121,36 @@ int spattn_pack_mask(void* packed, const int* booleanmask, int batch, int heads,
 int spattn_packedmask_to_indexmask(int* kv_indices, int* num_kv_indices, const void* packed, int batch, int heads,
                                    int seq, int seqblocks, int mask_stride, void* stream);
 
+/* The threshold sweep of booleanmask_128 (include/mask_utils.cuh:131-243) with a bit-packed
+ * result: one bit per (q-block, key), set where some row r of the q-block has
+ * softmax(r, key) > threshold and key < kv_len - the `> 0` view of the vote mask that every
+ * consumer of the reference takes (python/spattn/mask_utils.py:269, include/mask_utils.cuh:297),
+ * in the layout of `pack` (python/spattn/mask_utils.py:421-430; least significant bit first).
+ * qblk = 128: rows are the reference's 128-row q-blocks, packed is
+ * [batch,heads,ceil(seq/128),mask_stride/8] bytes and equals spattn_pack_mask of the vote mask.
+ * qblk = 64: one row per 64-row q-block, [batch,heads,ceil(seq/64),mask_stride/8]: the votes
+ * of the two halves of a 128-row block are kept apart (the lists a 64-row-q-block attention
+ * kernel needs).  Every word of every row is written; 1/32 of the bytes of the int32 mask. */
+int spattn_booleanmask_packed(void* packed, float threshold, int mask_stride, int qblk, const float* max_q,
+                              const float* denom, const void* q, const void* k, int batch, int heads, int seq, int D,
+                              int kv_len, float scale, void* stream);
+
+/* Key mask -> KV-block lists.  Key block J (keys 64J .. 64J+63) of a mask row is kept when one
+ * of its keys c < seq is set: MB[row,J] = OR_c M[row,c]  (the block form of
+ * booleanmask_to_indexmask, include/mask_utils.cuh:273-302; seq is the kv length).
+ * blk_indices int32 [batch,heads,seqblocks,max_blocks] receives the kept block ids of each row
+ * in ASCENDING order, entries behind them keep the caller's fill; blk_counts int32
+ * [batch,heads,seqblocks] the number of kept blocks (if it exceeds max_blocks only the first
+ * max_blocks ids are written; the attention entry points clamp a count to max_blocks).
+ * blockmask may be NULL, else uint8 [batch,heads,seqblocks,mask_stride/64] receives MB (0/1).
+ * The outputs feed spattn_sp_attn_blocks directly.  Sources: the bit-packed mask
+ * (seqblocks rows of mask_stride/8 bytes) or the int32 vote mask. */
+int spattn_packedmask_to_blocklists(int* blk_indices, int* blk_counts, void* blockmask, const void* packed, int batch,
+                                    int heads, int seq, int seqblocks, int mask_stride, int max_blocks, void* stream);
+int spattn_booleanmask_to_blocklists(int* blk_indices, int* blk_counts, void* blockmask, const int* booleanmask,
+                                     int batch, int heads, int seq, int seqblocks, int mask_stride, int max_blocks,
+                                     void* stream);
+
 /* Top-k mask generator (python/spattn/mask_utils.py:389-417, qk_topkmask_indices): per
  * q-block of `blocksz` rows the select_k keys c < kv_len (0 = seq) with the largest
  * (block mean of q / sqrt(D)) . k[c], every step rounded to bf16 as the reference's bf16 torch
@@ -140,7 +170,10 @@ int spattn_qk_topkmask_indices(int* kv_indices, int* num_kv_indices, void* score
  * flat q-block index of the count tensor): longest lists first, in quarter-octave classes of the
  * count, stable inside a class; if the longest list is less than twice the shortest, the default order.  The
  * _ordered forms of the two list-driven attention entry points let workgroup i take q-block
- * order[i]; results are bit-identical to the plain forms, only the schedule changes. */
+ * order[i]; results are bit-identical to the plain forms, only the schedule changes.
+ * order must be a permutation of 0..n-1: an entry outside that range is skipped by the kernel
+ * (nothing is read or written for it), a q-block that no entry names keeps whatever o held, and
+ * a q-block named twice is computed twice. */
 int spattn_qblock_order(int* order, const int* counts, int n, void* stream);
 int spattn_sp_attn_ordered(void* o, float* lse, const void* q, const void* k, const void* v, const int* kv_indices,
                            const int* num_kv_indices, const int* order, int mask_stride, int qblk, int batch, int heads,

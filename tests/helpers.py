@@ -15,22 +15,27 @@ def f32(t):
 def assert_close_o(got, want, what=""):
     got = np.asarray(got, np.float32)
     want = np.asarray(want, np.float32)
+    assert np.isfinite(want).all(), "%s: non-finite expected value (the checker itself is broken)" % what
     assert np.isfinite(got).all(), "%s: non-finite output" % what
     err = np.abs(got - want)
     lim = O_ATOL + O_RTOL * np.abs(want)
-    bad = err > lim
+    bad = ~(err <= lim)   # a NaN on either side fails
     assert not bad.any(), "%s: %d of %d outside tolerance, max err %.4g" % (what, bad.sum(), bad.size, err.max())
 
 
 def assert_close_stat(got, want, what="", rtol=STAT_RTOL, atol=1e-5):
     got = np.asarray(got, np.float64)
     want = np.asarray(want, np.float64)
-    same_inf = np.isinf(want) & (got == want)
-    err = np.abs(got - want)
-    lim = atol + rtol * np.abs(want)
-    bad = (err > lim) & ~same_inf
-    bad |= np.isnan(got)
-    assert not bad.any(), "%s: %d of %d outside tolerance, max err %.4g" % (what, bad.sum(), bad.size, np.nanmax(np.where(same_inf, 0, err)))
+    assert not np.isnan(want).any(), "%s: NaN in the expected value (the checker itself is broken)" % what
+    # infinities must agree in place and sign; everything else is compared where both are finite
+    inf_w, inf_g = np.isinf(want), np.isinf(got)
+    same_inf = inf_w & inf_g & (got == want)
+    fin = np.isfinite(want) & np.isfinite(got)
+    err = np.zeros(want.shape, np.float64)
+    err[fin] = np.abs(got[fin] - want[fin])
+    lim = atol + rtol * np.abs(np.where(fin, want, 0.0))
+    bad = ~(err <= lim) | ~(fin | same_inf)
+    assert not bad.any(), "%s: %d of %d outside tolerance, max err %.4g" % (what, bad.sum(), bad.size, err.max())
 
 
 def to_dev(dev, *ts):

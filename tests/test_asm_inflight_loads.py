@@ -4,7 +4,12 @@ vmcnt wait.  To the compiler those registers hold their values from the moment t
 statement ends, so nothing stops it from copying or spilling them while the load is still in
 flight.  This test compiles the three attention translation units to assembly (no GPU needed)
 and checks that between every such load and the first wait that covers it no other instruction
-names its destination registers."""
+names its destination registers.
+
+The HBM -> LDS copies set m0 inside their asm statement without telling the compiler (naming a
+reserved register as clobbered only draws a warning).  That is sound as long as the compiler
+itself never uses m0 in these kernels: the second check asserts that no instruction outside an
+asm statement names m0 in any translation unit that issues such copies."""
 import re
 import shutil
 import subprocess
@@ -17,6 +22,7 @@ from fgattn_tk_cuda_amd import build
 
 CSRC = Path(build.__file__).resolve().parent / "csrc"
 UNITS = ["attn_inst_blocks.hip", "attn_inst_tokens.hip", "attn_inst_dense.hip"]
+M0_UNITS = UNITS + ["mask_kernels.hip"]
 
 
 def _regs(text):
@@ -64,6 +70,29 @@ def inflight_accesses(listing):
     return found
 
 
+def m0_uses_outside_asm(listing):
+    """Lines outside ASMSTART/ASMEND blocks whose instruction names m0."""
+    found, inside = [], False
+    for n, raw in enumerate(listing.split("\n")):
+        if "#ASMSTART" in raw:
+            inside = True
+            continue
+        if "#ASMEND" in raw:
+            inside = False
+            continue
+        t = raw.split(";")[0].strip()
+        if not inside and t and not t.startswith(".") and re.search(r"\bm0\b", t):
+            found.append((n + 1, t))
+    return found
+
+
+def test_m0_checker_sees_a_compiler_use():
+    ok = "\t;;#ASMSTART\n\ts_mov_b32 m0, s3\n\tglobal_load_lds_dwordx4 v1, s[0:1]\n\t;;#ASMEND\n\tv_mov_b32_e32 v2, v3\n"
+    bad = ok + "\ts_mov_b32 m0, -1\n"
+    assert m0_uses_outside_asm(ok) == []
+    assert len(m0_uses_outside_asm(bad)) == 1
+
+
 def test_checker_sees_an_access_to_a_register_in_flight():
     bad = "\tglobal_load_dwordx4 v[4:7], v[2:3], off\n\tglobal_load_lds_dwordx4 v9, s[0:1]\n\tv_mov_b32_e32 v20, v5\n\ts_waitcnt vmcnt(0)\n"
     good = "\tglobal_load_dwordx4 v[4:7], v[2:3], off\n\tglobal_load_lds_dwordx4 v9, s[0:1]\n\ts_waitcnt vmcnt(1)\n\tv_mov_b32_e32 v20, v5\n"
@@ -81,9 +110,14 @@ def test_no_instruction_touches_a_register_with_a_load_in_flight(tmp_path):
                        check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
         return out.read_text()
 
-    with ThreadPoolExecutor(max_workers=3) as ex:
-        texts = list(ex.map(listing, UNITS))
-    for unit, text in zip(UNITS, texts):
+    with ThreadPoolExecutor(max_workers=4) as ex:
+        texts = list(ex.map(listing, M0_UNITS))
+    for unit, text in zip(M0_UNITS, texts):
+        assert "global_load_lds_dwordx4" in text, unit
+        uses = m0_uses_outside_asm(text)
+        assert not uses, "%s: the compiler uses m0 next to hand-written copies: %s" % (unit, uses[:3])
+        if unit not in UNITS:
+            continue
         assert "global_load_dword" in text, unit
         found = inflight_accesses(text)
         assert not found, "%s: %s" % (unit, found[:3])

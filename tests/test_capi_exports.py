@@ -22,7 +22,8 @@ def test_header_declares_expected_surface():
     for ref in ("attn_fwd_wg_impl", "attn_sparse_fwd_wg_impl", "allindex_mask_impl", "attn_maxq_denom_impl",
                 "maxq_denom_impl", "booleanmask_128_impl", "booleanmask_to_indexmask_impl"):
         assert ref in names
-    assert "spattn_sp_attn_blocks" in names and "spattn_packedmask_to_indexmask" in names and "spattn_qk_topkmask_indices" in names and "spattn_qblock_order" in names and len(names) == 24
+    assert "spattn_sp_attn_blocks" in names and "spattn_packedmask_to_indexmask" in names and "spattn_qk_topkmask_indices" in names and "spattn_qblock_order" in names
+    assert "spattn_booleanmask_packed" in names and "spattn_packedmask_to_blocklists" in names and "spattn_booleanmask_to_blocklists" in names
 
 
 def test_library_exports_every_declared_symbol():
@@ -54,6 +55,11 @@ def test_argument_checks_return_before_any_launch():
     assert lib.spattn_sp_attn(p16, None, p16, p16, p16, p16, p16, 128, 32, 1, 1, 128, 128, 0, 0.0, None) == -4
     assert lib.spattn_booleanmask_to_indexmask(p16, p16, p16, 1, 1, 10, 1, 100, None) == -3
     assert lib.spattn_all_index_mask(None, p16, 1, 1, 1, 1, 128, None) == -1
+    assert lib.spattn_full_attn(p16, None, p16, p16, p16, 1, 1, 1 << 24, 128, 0, 0.0, None) == -6
+    assert lib.spattn_booleanmask_packed(p16, 0.5, 128, 96, p16, p16, p16, p16, 1, 1, 128, 64, 0, 0.0, None) == -4
+    assert lib.spattn_booleanmask_packed(p16, 0.5, 64, 128, p16, p16, p16, p16, 1, 1, 128, 64, 0, 0.0, None) == -3
+    assert lib.spattn_packedmask_to_blocklists(p16, p16, None, p16, 1, 1, 10, 1, 128, 0, None) == -6
+    assert lib.spattn_booleanmask_to_blocklists(p16, p16, None, None, 1, 1, 10, 1, 128, 2, None) == -1
     # the reference-named wrappers record their status instead of returning it
     lib.attn_fwd_wg_impl(None, None, None, None, 1, 1, 128, 128)
     assert lib.spattn_last_status() == -1

@@ -184,10 +184,14 @@ def test_cfg4_shape_topk_generator_sampled_rows(dev):
 
 
 def test_cfg4_padded_threshold_pipeline(dev):
-    """N=32760 (padded to 32768), d=64, clustered keys: statistics -> vote mask -> index lists
-    -> sparse attention, two heads; each stage checked on sampled q-blocks."""
+    """B=1 H=24 N=32760 (padded to 32768), d=64, clustered keys: statistics -> vote mask -> index
+    lists -> sparse attention at the full head count.  The lists and counts of all 6144 mask rows
+    are compared bit for bit (more rows than one round of the compaction grid), the bit-packed
+    route must give the same lists, the other stages are checked on sampled q-blocks."""
     print("case cfg4 padded pipeline", flush=True)
-    B, H, S, D = 1, 2, 32760, 64
+    c = wl.CONFIGS["cfg4_threshold_padded"]
+    B, H, S, D = c["B"], c["H"], c["S"], c["D"]
+    assert (B, H, S, D) == (1, 24, 32760, 64)
     q, k, v = wl.clustered_qkv(B, H, S, D, seed=7)
     qd, kd, vd = to_dev(dev, q, k, v)
     Sp, SB = 32768, 256
@@ -196,7 +200,7 @@ def test_cfg4_padded_threshold_pipeline(dev):
     capi.maxq_denom(mx, dn, qd, kd)
     assert np.all(f32(mx)[..., S:] == 0) and np.all(np.isneginf(f32(dn)[..., S:]))
     rng = np.random.default_rng(8)
-    blocks = [(int(rng.integers(H)), int(rng.integers(SB))) for _ in range(4)] + [(0, SB - 1)]   # incl. the ragged block
+    blocks = [(int(rng.integers(H)), int(rng.integers(SB))) for _ in range(4)] + [(0, SB - 1), (H - 1, SB - 1)]   # incl. the ragged block
     kf = f32(k)
     for h, i in blocks:
         r = slice(i * 128, min(S, (i + 1) * 128))
@@ -205,26 +209,41 @@ def test_cfg4_padded_threshold_pipeline(dev):
         d = np.exp2((s - m[:, None]) * (orc.LOG2E / 8.0)).sum(1)
         assert_close_stat(f32(mx)[0, h, 0, r], m, "max_q", atol=1e-3)
         assert_close_stat(f32(dn)[0, h, 0, r], d, "denom")
-    # threshold: keep roughly 8 % of the (q-block, 64-key block) pairs of head 0, from sampled q-blocks
+    # threshold: keep about 8 % of the (q-block, 64-key block) pairs, from sampled q-blocks of three heads
     samp = []
-    for i in range(0, SB, 32):
-        r = slice(i * 128, min(S, (i + 1) * 128))
-        s = f32(q[0, 0, r]) @ kf[0, 0].T
-        p = np.exp2((s - f32(mx)[0, 0, 0, r, None]) * (orc.LOG2E / 8.0)) / f32(dn)[0, 0, 0, r, None]
-        pm = np.concatenate([p.max(0), np.zeros(Sp - S, np.float32)]).reshape(-1, 64).max(1)
-        samp.append(pm)
+    for h in (0, 11, 23):
+        for i in range(0, SB, 32):
+            r = slice(i * 128, min(S, (i + 1) * 128))
+            s = f32(q[0, h, r]) @ kf[0, h].T
+            p = np.exp2((s - f32(mx)[0, h, 0, r, None]) * (orc.LOG2E / 8.0)) / f32(dn)[0, h, 0, r, None]
+            pm = np.concatenate([p.max(0), np.zeros(Sp - S, np.float32)]).reshape(-1, 64).max(1)
+            samp.append(pm)
     thr = float(np.quantile(np.concatenate(samp), 0.92))
     mask = torch.zeros((B, H, SB, Sp), dtype=torch.int32, device=dev)
     capi.booleanmask_128(mask, mx, dn, qd, kd, thr)
     kvi = torch.full((B, H, SB, Sp), Sp, dtype=torch.int32, device=dev)
     kvn = torch.zeros((B, H, SB), dtype=torch.int32, device=dev)
     capi.booleanmask_to_indexmask(kvi, kvn, mask, S)
+    # the bit-packed route (mask cache) over the same 6144 rows
+    packed = torch.empty((B, H, SB, Sp // 8), dtype=torch.uint8, device=dev)
+    capi.pack_mask(packed, mask)
+    kvi2 = torch.full((B, H, SB, Sp), Sp, dtype=torch.int32, device=dev)
+    kvn2 = torch.zeros((B, H, SB), dtype=torch.int32, device=dev)
+    capi.packedmask_to_indexmask(kvi2, kvn2, packed, S)
+    assert torch.equal(kvi, kvi2) and torch.equal(kvn, kvn2)
+    del kvi2, kvn2
+    assert int(mask.min()) >= 0 and int(mask.max()) <= 8 and not bool(mask[..., S:].any())
+    blockmask = (mask > 0).view(B, H, SB, Sp // 64, 64).any(-1)
+    dens = float(blockmask.float().mean())
+    assert 0.06 < dens < 0.10, dens
+    per_head = blockmask.float().mean(dim=(0, 2, 3)).cpu().numpy()
+    assert per_head.min() > 0.04 and per_head.max() < 0.12, per_head
+    # all 6144 rows: counts, ascending lists, fill, bit for bit against the plain loop
     mh = mask.cpu().numpy()
-    assert mh.min() >= 0 and mh.max() <= 8 and np.all(mh[..., S:] == 0)
-    wi, wn = orc.booleanmask_to_indexmask(mh, S)                                   # bit-exact compaction
+    assert np.array_equal(np.unpackbits(packed.cpu().numpy(), axis=-1, bitorder="little"), (mh > 0).astype(np.uint8))
+    wi, wn = orc.booleanmask_to_indexmask(mh, S)
     assert np.array_equal(kvn.cpu().numpy(), wn) and np.array_equal(kvi.cpu().numpy(), wi)
-    blockmask = orc.block_mask_from_votes(mh[:, :1], S)
-    assert 0.02 < blockmask.mean() < 0.3, blockmask.mean()
+    assert np.array_equal(orc.block_mask_from_votes(mh[:, :2], S), blockmask[:, :2, :, : orc.ceil_div(S, 64)].cpu().numpy())
     for h, i in blocks:
         r = slice(i * 128, min(S, (i + 1) * 128))
         s = f32(q[0, h, r]) @ kf[0, h].T
@@ -232,6 +251,7 @@ def test_cfg4_padded_threshold_pipeline(dev):
         pmax = p.max(0)
         near = np.abs(pmax - thr) <= 1e-2 * thr
         assert np.array_equal((mh[0, h, i, :S] > 0) | near, (pmax > thr) | near), "mask row (%d,%d)" % (h, i)
+    del mh
     o = torch.full_like(qd, float("nan"))
     capi.sp_attn(o, qd, kd, vd, kvi, kvn)
     assert torch.isfinite(o.float()).all()

@@ -87,6 +87,53 @@ def test_packed_mask_round_trip_bit_exact(dev, SB, ms, seq, density):
     assert torch.equal(kvi, kvi2) and torch.equal(kvn, kvn2)
 
 
+def _run_mask(rng, shape, density):
+    """A 0..8 vote mask whose kept keys come in runs (what a threshold mask looks like)."""
+    B, H, SB, ms = shape
+    coarse = rng.random((B, H, SB, ms // 16)) < density
+    fine = rng.random((B, H, SB, ms)) < 0.7
+    keep = np.repeat(coarse, 16, axis=-1) & fine
+    return keep.astype(np.int32) * rng.integers(1, 9, size=shape, dtype=np.int32)
+
+
+def test_compaction_more_rows_than_one_round_of_the_grid(dev):
+    """5120 mask rows: the compaction kernel's persistent waves (1024 workgroups x 4 rows) take
+    a second row each; every list, count and fill value bit for bit."""
+    print("case compaction many rows", flush=True)
+    B, H, SB, ms, seq = 1, 40, 128, 256, 250
+    rng = np.random.default_rng(81)
+    mask = _run_mask(rng, (B, H, SB, ms), 0.12)
+    mask[0, 3, 5] = 0                      # an empty row
+    mask[0, 39, 127] = 1                   # a full row, the last one
+    md = torch.from_numpy(mask).to(dev)
+    kvi = torch.full((B, H, SB, ms), ms, dtype=torch.int32, device=dev)
+    kvn = torch.full((B, H, SB), -1, dtype=torch.int32, device=dev)
+    capi.booleanmask_to_indexmask(kvi, kvn, md, seq)
+    wi, wn = orc.booleanmask_to_indexmask(mask, seq)
+    assert np.array_equal(kvn.cpu().numpy(), wn)
+    assert np.array_equal(kvi.cpu().numpy(), wi)
+    assert wn[0, 3, 5] == 0 and wn[0, 39, 127] == seq
+
+
+def test_bit_kernels_more_rows_than_one_round_of_the_grid(dev):
+    """8960 mask rows: pack_mask and packedmask_to_indexmask both walk more than 8192 rows."""
+    print("case bit kernels many rows", flush=True)
+    B, H, SB, ms, seq = 1, 70, 128, 256, 256
+    rng = np.random.default_rng(82)
+    mask = _run_mask(rng, (B, H, SB, ms), 0.1)
+    mask[0, 69, 127] = 2
+    md = torch.from_numpy(mask).to(dev)
+    packed = torch.full((B, H, SB, ms // 8), 0x5A, dtype=torch.uint8, device=dev)
+    capi.pack_mask(packed, md)
+    assert np.array_equal(packed.cpu().numpy(), orc.pack_mask(mask))
+    kvi = torch.full((B, H, SB, ms), ms, dtype=torch.int32, device=dev)
+    kvn = torch.full((B, H, SB), -1, dtype=torch.int32, device=dev)
+    capi.packedmask_to_indexmask(kvi, kvn, packed, seq)
+    wi, wn = orc.booleanmask_to_indexmask(mask, seq)
+    assert np.array_equal(kvn.cpu().numpy(), wn)
+    assert np.array_equal(kvi.cpu().numpy(), wi)
+
+
 def test_all_index_mask(dev):
     print("case all_index_mask", flush=True)
     B, H, SB, S, ms = 2, 3, 5, 600, 640

@@ -51,6 +51,19 @@ def test_capi_rejects_host_tensors_without_touching_the_device():
         capi.full_attn(torch.zeros_like(q), q, q, q)
 
 
+def test_capi_rejects_a_work_order_of_the_wrong_size():
+    """A work order names every q-block once: one that is shorter (or longer) than the count
+    tensor never reaches the device."""
+    q = torch.zeros((1, 2, 256, 64), dtype=torch.bfloat16)
+    idx = torch.zeros((1, 2, 2, 256), dtype=torch.int32)
+    cnt = torch.zeros((1, 2, 2), dtype=torch.int32)
+    for bad in (torch.zeros(3, dtype=torch.int32), torch.zeros(5, dtype=torch.int32)):
+        with pytest.raises(ValueError, match="order"):
+            capi.sp_attn(q, q, q, q, idx, cnt, order=bad)
+        with pytest.raises(ValueError, match="order"):
+            capi.sp_attn_blocks(q, q, q, q, idx[..., :4].contiguous(), cnt, qblk=128, order=bad)
+
+
 def test_torch_mask_helpers_match_oracle():
     from fgattn_tk_cuda_amd.spattn import mask_utils as mu
 
