@@ -1,6 +1,9 @@
 // PyTorch operator binding: registers the seven ops of the reference extension in the
 // `cuda_attn` namespace (python/extension.cpp:81-358) and exposes the same seven functions
-// as a pybind module (python/extension.cpp:362-370).  Host code only: every op checks its
+// as a pybind module (python/extension.cpp:362-370).  Operators under further names carry what
+// the seven schemas cannot: a runtime kv length (the reference hard-codes one,
+// python/cuda_attn.cu:28-31), a softmax scale, a log-sum-exp output, KV-block lists, bit-packed
+// masks, and a work order computed once and reused.  Host code only: every op checks its
 // arguments and forwards raw device pointers to the C ABI of libspattn_hip.so on the
 // current HIP stream.  Unlike the reference, unsupported inputs raise instead of silently
 // returning (python/cuda_attn.cu:33-36 under -DNDEBUG).
@@ -46,17 +49,46 @@ int infer_qblk(int64_t seq, int64_t seqblocks) {
   return 0;
 }
 
+using OptTensor = c10::optional<torch::Tensor>;
+
+// optional fp32 [B,H,S] log-sum-exp output
+float* lse_ptr(const OptTensor& lse, const torch::Tensor& q) {
+  if (!lse.has_value() || !lse->defined()) return nullptr;
+  check_aux(*lse, "lse", at::kFloat, q);
+  TORCH_CHECK(lse->numel() == q.size(0) * q.size(1) * q.size(2), "lse must hold B*H*S floats");
+  return lse->data_ptr<float>();
+}
+
+// optional int32 work order with one entry per q-block
+const int* order_ptr(const OptTensor& order, const torch::Tensor& counts) {
+  if (!order.has_value() || !order->defined()) return nullptr;
+  check_aux(*order, "order", at::kInt, counts);
+  TORCH_CHECK(order->numel() == counts.numel(), "order must have one entry per q-block (B*H*SB)");
+  return order->data_ptr<int>();
+}
+
+int checked_kv_len(int64_t kv_len, const torch::Tensor& q) {
+  TORCH_CHECK(kv_len >= 0 && kv_len <= q.size(2), "kv_len must lie in [0, S] (0 = S)");
+  return (int)kv_len;
+}
+
 }  // namespace
 
-void full_attn(torch::Tensor o, torch::Tensor q, torch::Tensor k, torch::Tensor v) {
+void full_attn_ex(torch::Tensor o, OptTensor lse, torch::Tensor q, torch::Tensor k, torch::Tensor v, double scale,
+                  int64_t kv_len) {
   check_bhsd(q, "q", q);
   check_bhsd(k, "k", q);
   check_bhsd(v, "v", q);
   check_bhsd(o, "o", q);
   const DeviceGuard guard(q.device());
-  check_status(spattn_full_attn(o.data_ptr(), nullptr, q.data_ptr(), k.data_ptr(), v.data_ptr(), (int)q.size(0),
-                                (int)q.size(1), (int)q.size(2), (int)q.size(3), 0, 0.f, cur_stream()),
+  check_status(spattn_full_attn(o.data_ptr(), lse_ptr(lse, q), q.data_ptr(), k.data_ptr(), v.data_ptr(), (int)q.size(0),
+                                (int)q.size(1), (int)q.size(2), (int)q.size(3), checked_kv_len(kv_len, q), (float)scale,
+                                cur_stream()),
                "full_attn");
+}
+
+void full_attn(torch::Tensor o, torch::Tensor q, torch::Tensor k, torch::Tensor v) {
+  full_attn_ex(o, c10::nullopt, q, k, v, 0.0, 0);
 }
 
 void all_index_mask(torch::Tensor kv_indices, torch::Tensor kv_num_indices, int64_t batch, int64_t heads,
@@ -74,8 +106,28 @@ void all_index_mask(torch::Tensor kv_indices, torch::Tensor kv_num_indices, int6
                "all_index_mask");
 }
 
-void sp_attn(torch::Tensor o, torch::Tensor q, torch::Tensor k, torch::Tensor v, torch::Tensor kv_indices,
-             torch::Tensor kv_num_indices) {
+// Token lists.  order: the work order of spattn_qblock_order for these counts, or none.
+static void sp_attn_impl(torch::Tensor& o, const OptTensor& lse, torch::Tensor& q, torch::Tensor& k, torch::Tensor& v,
+                         torch::Tensor& kv_indices, torch::Tensor& kv_num_indices, const int* order, double scale,
+                         int64_t kv_len) {
+  const int qblk = infer_qblk(q.size(2), kv_indices.size(2));
+  const int B = (int)q.size(0), H = (int)q.size(1), S = (int)q.size(2), D = (int)q.size(3);
+  const int kv = checked_kv_len(kv_len, q);
+  if (order != nullptr) {
+    check_status(spattn_sp_attn_ordered(o.data_ptr(), lse_ptr(lse, q), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                        kv_indices.data_ptr<int>(), kv_num_indices.data_ptr<int>(), order,
+                                        (int)kv_indices.size(3), qblk, B, H, S, D, kv, (float)scale, cur_stream()),
+                 "sp_attn");
+  } else {
+    check_status(spattn_sp_attn(o.data_ptr(), lse_ptr(lse, q), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                kv_indices.data_ptr<int>(), kv_num_indices.data_ptr<int>(), (int)kv_indices.size(3), qblk,
+                                B, H, S, D, kv, (float)scale, cur_stream()),
+                 "sp_attn");
+  }
+}
+
+static void check_sp_attn_args(torch::Tensor& o, torch::Tensor& q, torch::Tensor& k, torch::Tensor& v,
+                               torch::Tensor& kv_indices, torch::Tensor& kv_num_indices) {
   check_bhsd(q, "q", q);
   check_bhsd(k, "k", q);
   check_bhsd(v, "v", q);
@@ -84,26 +136,82 @@ void sp_attn(torch::Tensor o, torch::Tensor q, torch::Tensor k, torch::Tensor v,
   check_aux(kv_num_indices, "kv_num_indices", at::kInt, q);
   TORCH_CHECK(kv_indices.dim() == 4 && kv_indices.size(0) == q.size(0) && kv_indices.size(1) == q.size(1),
               "kv_indices must be [B,H,SB,mask_stride]");
-  const int qblk = infer_qblk(q.size(2), kv_indices.size(2));
   // the reference does not check the shape of kv_num_indices, only its element order
   TORCH_CHECK(kv_num_indices.numel() == q.size(0) * q.size(1) * kv_indices.size(2), "kv_num_indices must have B*H*SB entries");
+}
+
+void sp_attn(torch::Tensor o, torch::Tensor q, torch::Tensor k, torch::Tensor v, torch::Tensor kv_indices,
+             torch::Tensor kv_num_indices) {
+  check_sp_attn_args(o, q, k, v, kv_indices, kv_num_indices);
   const DeviceGuard guard(q.device());
   // Threshold masks give lists of very different lengths: the q-blocks are handed to the
   // workgroups longest list first (the order is a small device tensor from torch's caching
-  // allocator; lists within a factor of two of each other keep the default order).
+  // allocator; lists within a factor of two of each other keep the default order).  Callers
+  // that reuse their lists compute the order once (qblock_order) and pass it to sp_attn_ex.
   torch::Tensor order = torch::empty({kv_num_indices.numel()}, kv_num_indices.options());
   check_status(spattn_qblock_order(order.data_ptr<int>(), kv_num_indices.data_ptr<int>(), (int)kv_num_indices.numel(),
                                    cur_stream()),
                "sp_attn (work order)");
-  check_status(spattn_sp_attn_ordered(o.data_ptr(), nullptr, q.data_ptr(), k.data_ptr(), v.data_ptr(),
-                                      kv_indices.data_ptr<int>(), kv_num_indices.data_ptr<int>(), order.data_ptr<int>(),
-                                      (int)kv_indices.size(3), qblk, (int)q.size(0), (int)q.size(1), (int)q.size(2),
-                                      (int)q.size(3), 0, 0.f, cur_stream()),
-               "sp_attn");
+  sp_attn_impl(o, c10::nullopt, q, k, v, kv_indices, kv_num_indices, order.data_ptr<int>(), 0.0, 0);
 }
 
-void fullattn_maxq_denom(torch::Tensor o, torch::Tensor o_max_q, torch::Tensor o_denom, torch::Tensor q, torch::Tensor k,
-                         torch::Tensor v) {
+// sp_attn with an optional log-sum-exp output, an optional precomputed work order (none: the
+// default order, one launch and no allocation), a softmax scale (0 = 1/sqrt(D)) and a kv length.
+void sp_attn_ex(torch::Tensor o, OptTensor lse, torch::Tensor q, torch::Tensor k, torch::Tensor v,
+                torch::Tensor kv_indices, torch::Tensor kv_num_indices, OptTensor order, double scale, int64_t kv_len) {
+  check_sp_attn_args(o, q, k, v, kv_indices, kv_num_indices);
+  const DeviceGuard guard(q.device());
+  sp_attn_impl(o, lse, q, k, v, kv_indices, kv_num_indices, order_ptr(order, kv_num_indices), scale, kv_len);
+}
+
+// Sparse attention over lists of 64-key blocks: blk_idx int32 [B,H,ceil(S/qblk),max_blocks],
+// blk_cnt int32 with B*H*ceil(S/qblk) entries, qblk 64 or 128 (0 = implied by blk_idx.size(2)).
+void sp_attn_block(torch::Tensor o, OptTensor lse, torch::Tensor q, torch::Tensor k, torch::Tensor v,
+                   torch::Tensor blk_idx, torch::Tensor blk_cnt, OptTensor order, int64_t qblk, double scale,
+                   int64_t kv_len) {
+  check_bhsd(q, "q", q);
+  check_bhsd(k, "k", q);
+  check_bhsd(v, "v", q);
+  check_bhsd(o, "o", q);
+  check_aux(blk_idx, "blk_idx", at::kInt, q);
+  check_aux(blk_cnt, "blk_cnt", at::kInt, q);
+  TORCH_CHECK(blk_idx.dim() == 4 && blk_idx.size(0) == q.size(0) && blk_idx.size(1) == q.size(1),
+              "blk_idx must be [B,H,SB,max_blocks]");
+  if (qblk == 0) qblk = infer_qblk(q.size(2), blk_idx.size(2));
+  TORCH_CHECK(qblk == 64 || qblk == 128, "qblk must be 64 or 128");
+  TORCH_CHECK(blk_idx.size(2) == (q.size(2) + qblk - 1) / qblk, "blk_idx must hold ceil(S/qblk) lists per head");
+  TORCH_CHECK(blk_cnt.numel() == q.size(0) * q.size(1) * blk_idx.size(2), "blk_cnt must have B*H*SB entries");
+  const DeviceGuard guard(q.device());
+  const int B = (int)q.size(0), H = (int)q.size(1), S = (int)q.size(2), D = (int)q.size(3);
+  const int kv = checked_kv_len(kv_len, q);
+  const int* ord = order_ptr(order, blk_cnt);
+  if (ord != nullptr) {
+    check_status(spattn_sp_attn_blocks_ordered(o.data_ptr(), lse_ptr(lse, q), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                               blk_idx.data_ptr<int>(), blk_cnt.data_ptr<int>(), ord,
+                                               (int)blk_idx.size(3), (int)qblk, B, H, S, D, kv, (float)scale,
+                                               cur_stream()),
+                 "sp_attn_block");
+  } else {
+    check_status(spattn_sp_attn_blocks(o.data_ptr(), lse_ptr(lse, q), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                       blk_idx.data_ptr<int>(), blk_cnt.data_ptr<int>(), (int)blk_idx.size(3), (int)qblk,
+                                       B, H, S, D, kv, (float)scale, cur_stream()),
+                 "sp_attn_block");
+  }
+}
+
+// order int32 [n] <- the q-blocks of counts (int32, n entries) longest list first.
+void qblock_order(torch::Tensor order, torch::Tensor counts) {
+  TORCH_CHECK(counts.is_cuda() && counts.scalar_type() == at::kInt && counts.is_contiguous(),
+              "counts must be a contiguous int32 device tensor");
+  check_aux(order, "order", at::kInt, counts);
+  TORCH_CHECK(order.numel() == counts.numel() && counts.numel() > 0, "order must have one entry per count");
+  const DeviceGuard guard(counts.device());
+  check_status(spattn_qblock_order(order.data_ptr<int>(), counts.data_ptr<int>(), (int)counts.numel(), cur_stream()),
+               "qblock_order");
+}
+
+void fullattn_maxq_denom_ex(torch::Tensor o, torch::Tensor o_max_q, torch::Tensor o_denom, torch::Tensor q,
+                            torch::Tensor k, torch::Tensor v, double scale, int64_t kv_len) {
   check_bhsd(q, "q", q);
   check_bhsd(k, "k", q);
   check_bhsd(v, "v", q);
@@ -115,11 +223,17 @@ void fullattn_maxq_denom(torch::Tensor o, torch::Tensor o_max_q, torch::Tensor o
   const DeviceGuard guard(q.device());
   check_status(spattn_fullattn_maxq_denom(o.data_ptr(), o_max_q.data_ptr<float>(), o_denom.data_ptr<float>(), q.data_ptr(),
                                           k.data_ptr(), v.data_ptr(), (int)q.size(0), (int)q.size(1), (int)q.size(2),
-                                          (int)q.size(3), 0, 0.f, cur_stream()),
+                                          (int)q.size(3), checked_kv_len(kv_len, q), (float)scale, cur_stream()),
                "fullattn_maxq_denom");
 }
 
-void maxq_denom(torch::Tensor o_max_q, torch::Tensor o_denom, torch::Tensor q, torch::Tensor k) {
+void fullattn_maxq_denom(torch::Tensor o, torch::Tensor o_max_q, torch::Tensor o_denom, torch::Tensor q, torch::Tensor k,
+                         torch::Tensor v) {
+  fullattn_maxq_denom_ex(o, o_max_q, o_denom, q, k, v, 0.0, 0);
+}
+
+void maxq_denom_ex(torch::Tensor o_max_q, torch::Tensor o_denom, torch::Tensor q, torch::Tensor k, double scale,
+                   int64_t kv_len) {
   check_bhsd(q, "q", q);
   check_bhsd(k, "k", q);
   check_aux(o_max_q, "o_max_q", at::kFloat, q);
@@ -128,12 +242,17 @@ void maxq_denom(torch::Tensor o_max_q, torch::Tensor o_denom, torch::Tensor q, t
   TORCH_CHECK(o_max_q.numel() == need && o_denom.numel() == need, "o_max_q / o_denom must be [B,H,1,128*ceil(S/128)]");
   const DeviceGuard guard(q.device());
   check_status(spattn_maxq_denom(o_max_q.data_ptr<float>(), o_denom.data_ptr<float>(), q.data_ptr(), k.data_ptr(),
-                                 (int)q.size(0), (int)q.size(1), (int)q.size(2), (int)q.size(3), 0, 0.f, cur_stream()),
+                                 (int)q.size(0), (int)q.size(1), (int)q.size(2), (int)q.size(3), checked_kv_len(kv_len, q),
+                                 (float)scale, cur_stream()),
                "maxq_denom");
 }
 
-void booleanmask_128(torch::Tensor booleanmask, torch::Tensor o_max_q, torch::Tensor o_denom, torch::Tensor q,
-                     torch::Tensor k, double threshold) {
+void maxq_denom(torch::Tensor o_max_q, torch::Tensor o_denom, torch::Tensor q, torch::Tensor k) {
+  maxq_denom_ex(o_max_q, o_denom, q, k, 0.0, 0);
+}
+
+void booleanmask_128_ex(torch::Tensor booleanmask, torch::Tensor o_max_q, torch::Tensor o_denom, torch::Tensor q,
+                        torch::Tensor k, double threshold, double scale, int64_t kv_len) {
   check_bhsd(q, "q", q);
   check_bhsd(k, "k", q);
   check_aux(booleanmask, "booleanmask", at::kInt, q);
@@ -147,8 +266,82 @@ void booleanmask_128(torch::Tensor booleanmask, torch::Tensor o_max_q, torch::Te
   const DeviceGuard guard(q.device());
   check_status(spattn_booleanmask_128(booleanmask.data_ptr<int>(), (float)threshold, (int)booleanmask.size(3),
                                       o_max_q.data_ptr<float>(), o_denom.data_ptr<float>(), q.data_ptr(), k.data_ptr(),
-                                      (int)q.size(0), (int)q.size(1), (int)q.size(2), (int)q.size(3), 0, 0.f, cur_stream()),
+                                      (int)q.size(0), (int)q.size(1), (int)q.size(2), (int)q.size(3),
+                                      checked_kv_len(kv_len, q), (float)scale, cur_stream()),
                "booleanmask_128");
+}
+
+void booleanmask_128(torch::Tensor booleanmask, torch::Tensor o_max_q, torch::Tensor o_denom, torch::Tensor q,
+                     torch::Tensor k, double threshold) {
+  booleanmask_128_ex(booleanmask, o_max_q, o_denom, q, k, threshold, 0.0, 0);
+}
+
+// The threshold sweep with a bit-packed result: packed uint8 [B,H,ceil(S/qblk),mask_stride/8],
+// one bit per (q-block of qblk rows, key), least significant bit first.
+void booleanmask_packed(torch::Tensor packed, torch::Tensor o_max_q, torch::Tensor o_denom, torch::Tensor q,
+                        torch::Tensor k, double threshold, int64_t qblk, double scale, int64_t kv_len) {
+  check_bhsd(q, "q", q);
+  check_bhsd(k, "k", q);
+  check_aux(packed, "packed", at::kByte, q);
+  check_aux(o_max_q, "o_max_q", at::kFloat, q);
+  check_aux(o_denom, "o_denom", at::kFloat, q);
+  TORCH_CHECK(qblk == 64 || qblk == 128, "qblk must be 64 or 128");
+  TORCH_CHECK(packed.dim() == 4 && packed.size(0) == q.size(0) && packed.size(1) == q.size(1) &&
+                  packed.size(2) == (q.size(2) + qblk - 1) / qblk,
+              "packed must be [B,H,ceil(S/qblk),mask_stride/8]");
+  const int64_t need = q.size(0) * q.size(1) * padded128(q.size(2));
+  TORCH_CHECK(o_max_q.numel() == need && o_denom.numel() == need, "o_max_q / o_denom must be [B,H,1,128*ceil(S/128)]");
+  const DeviceGuard guard(q.device());
+  check_status(spattn_booleanmask_packed(packed.data_ptr(), (float)threshold, (int)packed.size(3) * 8, (int)qblk,
+                                         o_max_q.data_ptr<float>(), o_denom.data_ptr<float>(), q.data_ptr(), k.data_ptr(),
+                                         (int)q.size(0), (int)q.size(1), (int)q.size(2), (int)q.size(3),
+                                         checked_kv_len(kv_len, q), (float)scale, cur_stream()),
+               "booleanmask_packed");
+}
+
+// Key mask -> ascending lists of kept 64-key blocks (+ counts, + optional uint8 block mask
+// [B,H,SB,mask_stride/64]); the source is the bit-packed mask or the int32 vote mask.
+static void blocklists_common(torch::Tensor& blk_idx, torch::Tensor& blk_cnt, const OptTensor& blockmask,
+                              const torch::Tensor& src, int64_t mask_stride, int64_t seq) {
+  check_aux(blk_idx, "blk_idx", at::kInt, src);
+  check_aux(blk_cnt, "blk_cnt", at::kInt, src);
+  TORCH_CHECK(blk_idx.dim() == 4 && blk_idx.size(0) == src.size(0) && blk_idx.size(1) == src.size(1) &&
+                  blk_idx.size(2) == src.size(2) && blk_idx.size(3) > 0,
+              "blk_idx must be [B,H,SB,max_blocks]");
+  TORCH_CHECK(blk_cnt.numel() == src.size(0) * src.size(1) * src.size(2), "blk_cnt must have B*H*SB entries");
+  TORCH_CHECK(seq >= 0, "seq must not be negative");
+  if (blockmask.has_value() && blockmask->defined()) {
+    check_aux(*blockmask, "blockmask", at::kByte, src);
+    TORCH_CHECK(blockmask->numel() == blk_cnt.numel() * (mask_stride / 64), "blockmask must be uint8 [B,H,SB,mask_stride/64]");
+  }
+}
+
+void packedmask_to_blocklists(torch::Tensor blk_idx, torch::Tensor blk_cnt, OptTensor blockmask, torch::Tensor packed,
+                              int64_t seq) {
+  TORCH_CHECK(packed.is_cuda() && packed.scalar_type() == at::kByte && packed.is_contiguous() && packed.dim() == 4,
+              "packed must be a contiguous uint8 device tensor [B,H,SB,mask_stride/8]");
+  blocklists_common(blk_idx, blk_cnt, blockmask, packed, packed.size(3) * 8, seq);
+  const DeviceGuard guard(packed.device());
+  void* bm = (blockmask.has_value() && blockmask->defined()) ? blockmask->data_ptr() : nullptr;
+  check_status(spattn_packedmask_to_blocklists(blk_idx.data_ptr<int>(), blk_cnt.data_ptr<int>(), bm, packed.data_ptr(),
+                                               (int)packed.size(0), (int)packed.size(1), (int)seq, (int)packed.size(2),
+                                               (int)packed.size(3) * 8, (int)blk_idx.size(3), cur_stream()),
+               "packedmask_to_blocklists");
+}
+
+void booleanmask_to_blocklists(torch::Tensor blk_idx, torch::Tensor blk_cnt, OptTensor blockmask,
+                               torch::Tensor booleanmask, int64_t seq) {
+  TORCH_CHECK(booleanmask.is_cuda() && booleanmask.scalar_type() == at::kInt && booleanmask.is_contiguous() &&
+                  booleanmask.dim() == 4,
+              "booleanmask must be a contiguous int32 device tensor [B,H,SB,mask_stride]");
+  blocklists_common(blk_idx, blk_cnt, blockmask, booleanmask, booleanmask.size(3), seq);
+  const DeviceGuard guard(booleanmask.device());
+  void* bm = (blockmask.has_value() && blockmask->defined()) ? blockmask->data_ptr() : nullptr;
+  check_status(spattn_booleanmask_to_blocklists(blk_idx.data_ptr<int>(), blk_cnt.data_ptr<int>(), bm,
+                                                booleanmask.data_ptr<int>(), (int)booleanmask.size(0),
+                                                (int)booleanmask.size(1), (int)seq, (int)booleanmask.size(2),
+                                                (int)booleanmask.size(3), (int)blk_idx.size(3), cur_stream()),
+               "booleanmask_to_blocklists");
 }
 
 void booleanmask_to_indexmask(torch::Tensor kv_indices, torch::Tensor kv_numindices, torch::Tensor booleanmask, int64_t seq) {
@@ -242,6 +435,17 @@ void noop_mask(torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch
 void noop_b2i(torch::Tensor, torch::Tensor, torch::Tensor, int64_t) {}
 void noop2(torch::Tensor, torch::Tensor) {}
 void noop_topk(torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, int64_t, int64_t) {}
+void noop_full_ex(torch::Tensor, OptTensor, torch::Tensor, torch::Tensor, torch::Tensor, double, int64_t) {}
+void noop_sp_ex(torch::Tensor, OptTensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, OptTensor,
+                double, int64_t) {}
+void noop_sp_block(torch::Tensor, OptTensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+                   OptTensor, int64_t, double, int64_t) {}
+void noop_fmd_ex(torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, double, int64_t) {}
+void noop_md_ex(torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, double, int64_t) {}
+void noop_mask_ex(torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, double, double, int64_t) {}
+void noop_mask_packed(torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, double, int64_t, double,
+                      int64_t) {}
+void noop_blocklists(torch::Tensor, torch::Tensor, OptTensor, torch::Tensor, int64_t) {}
 
 TORCH_LIBRARY_FRAGMENT(cuda_attn, m) {
   m.def("full_attn(Tensor(a!) o, Tensor q, Tensor k, Tensor v) -> ()");
@@ -254,6 +458,17 @@ TORCH_LIBRARY_FRAGMENT(cuda_attn, m) {
   m.def("pack_mask(Tensor(a!) packed, Tensor booleanmask) -> ()");
   m.def("packedmask_to_indexmask(Tensor(a!) kv_indices, Tensor(b!) kv_numindices, Tensor packed, int seq) -> ()");
   m.def("qk_topkmask_indices(Tensor(a!) kv_indices, Tensor(b!) kv_numindices, Tensor(c!) score, Tensor(d!) qmean, Tensor q, Tensor k, int select_k, int blocksz) -> ()");
+  // scale 0 = 1/sqrt(D); kv_len 0 = S
+  m.def("full_attn_ex(Tensor(a!) o, Tensor(b!)? lse, Tensor q, Tensor k, Tensor v, float scale, int kv_len) -> ()");
+  m.def("sp_attn_ex(Tensor(a!) o, Tensor(b!)? lse, Tensor q, Tensor k, Tensor v, Tensor kv_indices, Tensor kv_num_indices, Tensor? order, float scale, int kv_len) -> ()");
+  m.def("sp_attn_block(Tensor(a!) o, Tensor(b!)? lse, Tensor q, Tensor k, Tensor v, Tensor blk_idx, Tensor blk_cnt, Tensor? order, int qblk, float scale, int kv_len) -> ()");
+  m.def("fullattn_maxq_denom_ex(Tensor(a!) o, Tensor(b!) o_max_q, Tensor(c!) o_denom, Tensor q, Tensor k, Tensor v, float scale, int kv_len) -> ()");
+  m.def("maxq_denom_ex(Tensor(a!) o_max_q, Tensor(b!) o_denom, Tensor q, Tensor k, float scale, int kv_len) -> ()");
+  m.def("booleanmask_128_ex(Tensor(a!) booleanmask, Tensor o_max_q, Tensor o_denom, Tensor q, Tensor k, float threshold, float scale, int kv_len) -> ()");
+  m.def("booleanmask_packed(Tensor(a!) packed, Tensor o_max_q, Tensor o_denom, Tensor q, Tensor k, float threshold, int qblk, float scale, int kv_len) -> ()");
+  m.def("packedmask_to_blocklists(Tensor(a!) blk_idx, Tensor(b!) blk_cnt, Tensor(c!)? blockmask, Tensor packed, int seq) -> ()");
+  m.def("booleanmask_to_blocklists(Tensor(a!) blk_idx, Tensor(b!) blk_cnt, Tensor(c!)? blockmask, Tensor booleanmask, int seq) -> ()");
+  m.def("qblock_order(Tensor(a!) order, Tensor counts) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(cuda_attn, Meta, m) {
@@ -267,6 +482,16 @@ TORCH_LIBRARY_IMPL(cuda_attn, Meta, m) {
   m.impl("pack_mask", noop2);
   m.impl("packedmask_to_indexmask", noop_b2i);
   m.impl("qk_topkmask_indices", noop_topk);
+  m.impl("full_attn_ex", noop_full_ex);
+  m.impl("sp_attn_ex", noop_sp_ex);
+  m.impl("sp_attn_block", noop_sp_block);
+  m.impl("fullattn_maxq_denom_ex", noop_fmd_ex);
+  m.impl("maxq_denom_ex", noop_md_ex);
+  m.impl("booleanmask_128_ex", noop_mask_ex);
+  m.impl("booleanmask_packed", noop_mask_packed);
+  m.impl("packedmask_to_blocklists", noop_blocklists);
+  m.impl("booleanmask_to_blocklists", noop_blocklists);
+  m.impl("qblock_order", noop2);
 }
 
 // The CUDA dispatch key serves HIP tensors on PyTorch-ROCm.
@@ -281,6 +506,16 @@ TORCH_LIBRARY_IMPL(cuda_attn, CUDA, m) {
   m.impl("pack_mask", pack_mask);
   m.impl("packedmask_to_indexmask", packedmask_to_indexmask);
   m.impl("qk_topkmask_indices", qk_topkmask_indices);
+  m.impl("full_attn_ex", full_attn_ex);
+  m.impl("sp_attn_ex", sp_attn_ex);
+  m.impl("sp_attn_block", sp_attn_block);
+  m.impl("fullattn_maxq_denom_ex", fullattn_maxq_denom_ex);
+  m.impl("maxq_denom_ex", maxq_denom_ex);
+  m.impl("booleanmask_128_ex", booleanmask_128_ex);
+  m.impl("booleanmask_packed", booleanmask_packed);
+  m.impl("packedmask_to_blocklists", packedmask_to_blocklists);
+  m.impl("booleanmask_to_blocklists", booleanmask_to_blocklists);
+  m.impl("qblock_order", qblock_order);
 }
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -294,4 +529,14 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("pack_mask", &pack_mask, "pack_mask");
   m.def("packedmask_to_indexmask", &packedmask_to_indexmask, "packedmask_to_indexmask");
   m.def("qk_topkmask_indices", &qk_topkmask_indices, "qk_topkmask_indices");
+  m.def("full_attn_ex", &full_attn_ex, "full_attn with lse, scale, kv_len");
+  m.def("sp_attn_ex", &sp_attn_ex, "sp_attn with lse, work order, scale, kv_len");
+  m.def("sp_attn_block", &sp_attn_block, "sparse attention over KV-block lists");
+  m.def("fullattn_maxq_denom_ex", &fullattn_maxq_denom_ex, "fullattn_maxq_denom with scale, kv_len");
+  m.def("maxq_denom_ex", &maxq_denom_ex, "maxq_denom with scale, kv_len");
+  m.def("booleanmask_128_ex", &booleanmask_128_ex, "booleanmask_128 with scale, kv_len");
+  m.def("booleanmask_packed", &booleanmask_packed, "threshold sweep, bit-packed result");
+  m.def("packedmask_to_blocklists", &packedmask_to_blocklists, "bit-packed mask -> KV-block lists");
+  m.def("booleanmask_to_blocklists", &booleanmask_to_blocklists, "vote mask -> KV-block lists");
+  m.def("qblock_order", &qblock_order, "work order, longest list first");
 }

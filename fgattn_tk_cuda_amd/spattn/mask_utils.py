@@ -16,20 +16,30 @@ from . import cuda_attn  # noqa: F401  (loading it registers torch.ops.cuda_attn
 spattn_interface = torch.ops.cuda_attn
 
 BLOCKSZ = 128   # q-block of the threshold pre-pass (python/spattn/mask_utils.py:249,312)
+BLOCKSZ_DEFAULT = BLOCKSZ
 
 
 def _padded(seq: int, blk: int = BLOCKSZ) -> int:
     return blk * ((seq + blk - 1) // blk)
 
 
+def _is_dev(t) -> bool:
+    return isinstance(t, torch.Tensor) and t.is_cuda
+
+
 # ----------------------------------------------------------------------------------
 # mask caches (python/spattn/mask_utils.py:17-98)
 # ----------------------------------------------------------------------------------
 class NaiveMaskCache:
-    """Index lists per layer, recomputed on the diffusion steps in ``compute_cache_at``."""
+    """Index lists per layer, recomputed on the diffusion steps in ``compute_cache_at``.
+
+    Next to the lists the cache keeps their work order (a function of the counts alone, see
+    ``qblock_order_cuda``): it is computed when the lists are stored, so a step that reuses
+    them is a single kernel launch.  ``get_order`` returns it (None for host tensors)."""
 
     def __init__(self, compute_cache_at):
         self.cache = {}
+        self.order = {}
         self.compute_cache_at = compute_cache_at
 
     def run_fullattn(self, ditrun):
@@ -38,8 +48,18 @@ class NaiveMaskCache:
     def get_mask_from_cache(self, layer):
         return self.cache[layer]
 
+    def get_order(self, layer):
+        return self.order.get(layer)
+
     def update_cache(self, layer, kv_indices, kv_num_indices):
         self.cache[layer] = (kv_indices, kv_num_indices)
+        self.order[layer] = qblock_order_cuda(kv_num_indices) if _is_dev(kv_num_indices) else None
+
+
+class BlockListCache(NaiveMaskCache):
+    """KV-block lists ([B,H,ceil(S/qblk),max_blocks] ids of 64-key blocks, counts) per layer, for
+    ``sp_attn_block``; same protocol as NaiveMaskCache.  No counterpart in the reference, whose
+    lists are per key."""
 
 
 class OffloadMaskCache(NaiveMaskCache):
@@ -253,23 +273,112 @@ def qk_indexmask_cuda(q, k, thresh, blocksz=128):
     return qk_indexmask_from_maxq_denom_cuda(max_q, denom, q, k, thresh, blocksz)
 
 
+def qblock_order_cuda(counts):
+    """int32 [counts.numel()]: the q-blocks longest list first (the schedule of the list-driven
+    attention operators); lists within a factor of two of each other keep the default order."""
+    order = torch.empty((counts.numel(),), dtype=torch.int32, device=counts.device)
+    spattn_interface.qblock_order(order, counts.contiguous())
+    return order
+
+
+# ----------------------------------------------------------------------------------
+# KV-block lists: the threshold mask at the granularity of 64-key blocks.  The sweep writes
+# one bit per (q-block, key) instead of an int32 vote count, and the lists hold block ids.
+# ----------------------------------------------------------------------------------
+KVBLK = 64
+
+
+def qk_packedmask_from_maxq_denom_cuda(max_q, denom, q, k, thresh, qblk=128, kv_len=0):
+    """uint8 [B,H,ceil(S/qblk),Sp/8], bit (c & 7) of byte c >> 3: some row of the q-block has
+    softmax(row, c) > thresh.  For qblk = 128 equal to ``pack(qk_bitmask_from_maxq_denom_cuda(...) > 0)``."""
+    B, H, S, _ = q.shape
+    packed = torch.empty((B, H, (S + qblk - 1) // qblk, max_q.shape[3] // 8), dtype=torch.uint8, device=q.device)
+    spattn_interface.booleanmask_packed(packed, max_q.contiguous(), denom.contiguous(), q.contiguous(), k.contiguous(),
+                                        thresh, qblk, 0.0, kv_len)
+    return packed
+
+
+def packedmask_to_blocklists_cuda(packed, seq=None, max_blocks=None, with_blockmask=False):
+    """Ascending lists of the 64-key blocks with a set key c < seq, padded with -1, and counts;
+    optionally the block mask uint8 [B,H,SB,mask_stride/64] as a third result."""
+    B, H, SB, MB = packed.shape
+    nb = MB * 8 // KVBLK
+    if seq is None:
+        seq = MB * 8
+    if max_blocks is None:
+        max_blocks = nb
+    blk_idx = torch.full((B, H, SB, max_blocks), -1, dtype=torch.int32, device=packed.device)
+    blk_cnt = torch.zeros((B, H, SB), dtype=torch.int32, device=packed.device)
+    blockmask = torch.empty((B, H, SB, nb), dtype=torch.uint8, device=packed.device) if with_blockmask else None
+    spattn_interface.packedmask_to_blocklists(blk_idx, blk_cnt, blockmask, packed.contiguous(), seq)
+    return (blk_idx, blk_cnt, blockmask) if with_blockmask else (blk_idx, blk_cnt)
+
+
+def bitmask_to_blocklists_cuda(booleanmask, seq=None, max_blocks=None, with_blockmask=False):
+    """The same from the int32 vote mask [B,H,SB,mask_stride]."""
+    B, H, SB, MS = booleanmask.shape
+    nb = MS // KVBLK
+    if seq is None:
+        seq = MS
+    if max_blocks is None:
+        max_blocks = nb
+    blk_idx = torch.full((B, H, SB, max_blocks), -1, dtype=torch.int32, device=booleanmask.device)
+    blk_cnt = torch.zeros((B, H, SB), dtype=torch.int32, device=booleanmask.device)
+    blockmask = torch.empty((B, H, SB, nb), dtype=torch.uint8, device=booleanmask.device) if with_blockmask else None
+    spattn_interface.booleanmask_to_blocklists(blk_idx, blk_cnt, blockmask, booleanmask.to(torch.int32).contiguous(), seq)
+    return (blk_idx, blk_cnt, blockmask) if with_blockmask else (blk_idx, blk_cnt)
+
+
+def qk_blocklists_from_maxq_denom_cuda(max_q, denom, q, k, thresh, qblk=128, kv_len=0):
+    """Row statistics -> bit-packed threshold mask -> KV-block lists for q-blocks of qblk rows."""
+    packed = qk_packedmask_from_maxq_denom_cuda(max_q, denom, q, k, thresh, qblk, kv_len)
+    return packedmask_to_blocklists_cuda(packed, kv_len or q.shape[2])
+
+
+def qk_blocklists_cuda(q, k, thresh, qblk=128, kv_len=0):
+    """Statistics sweep -> threshold sweep -> KV-block lists (the block form of qk_indexmask_cuda)."""
+    max_q, denom = _stats_buffers(q)
+    spattn_interface.maxq_denom_ex(max_q, denom, q.contiguous(), k.contiguous(), 0.0, kv_len)
+    return qk_blocklists_from_maxq_denom_cuda(max_q, denom, q, k, thresh, qblk, kv_len)
+
+
+def qk_blocklists(q, k, thresh=0.001, qblk=128):
+    """Pure-torch definition of the block lists: block J of q-block I is kept when some row of I
+    and some key of J have softmax > thresh.  Returns (blk_idx padded with -1, blk_cnt, blockmask)."""
+    B, H, S, _ = q.shape
+    m = qk_bitmask(q, k, thresh, qblk)                                   # [B,H,nq,S]
+    pad = (-S) % KVBLK
+    if pad:
+        m = torch.cat([m, torch.zeros((*m.shape[:3], pad), dtype=m.dtype, device=m.device)], dim=-1)
+    bm = m.view(*m.shape[:3], -1, KVBLK).any(dim=-1)
+    nq, nb = bm.shape[2], bm.shape[3]
+    idx, cnt = boolean_to_index_mask_2d(bm.reshape(B * H * nq, nb))
+    idx = torch.where(idx == nb, torch.full_like(idx, -1), idx)
+    return idx.view(B, H, nq, nb), cnt.view(B, H, nq), bm
+
+
 def qk_lshmask_indices(query, key, thresh, blocksz=128):
     raise NotImplementedError   # as in the reference (python/spattn/mask_utils.py:385-386)
 
 
-def qk_topkmask_indices(q, k, select_k, blocksz=128):
-    """Top-k keys per q-block by (block-mean query) . key (python/spattn/mask_utils.py:389-417)."""
-    B, H, S, D = q.shape
-    nb = (S + blocksz - 1) // blocksz
-    pad = nb * blocksz - S
-    qf = q.float()
-    if pad:
-        qf = torch.cat([qf, torch.zeros((B, H, pad, D), device=q.device)], dim=2)
-    rows = torch.full((nb,), float(blocksz), device=q.device)
-    rows[-1] = blocksz - pad
-    qmean = qf.view(B, H, nb, blocksz, D).sum(dim=3) / rows[None, None, :, None]
-    score = torch.einsum("bhmd,bhnd->bhmn", qmean * (D ** -0.5), k.float())
+def qk_topkmask_indices(q, k, select_k, B=None, H=None, S=None, D=None, BLOCKSZ=None, blocksz=None):
+    """Top-k keys per q-block by (block-mean query / sqrt(D)) . key, in the dtype of q like the
+    reference (python/spattn/mask_utils.py:389-417).  Takes the reference's positional form
+    ``(q, k, select_k, B, H, S, D, BLOCKSZ)`` as well as ``blocksz=`` alone, which is how the
+    reference's own caller passes it (python/spattn/sparseattn_functionals.py:46); sizes that
+    are not given are read from q."""
+    B, H, S, D = (int(x) if x is not None else int(d) for x, d in zip((B, H, S, D), q.shape))
+    blk = int(BLOCKSZ if BLOCKSZ is not None else (blocksz if blocksz is not None else BLOCKSZ_DEFAULT))
+    nfull = S // blk
+    parts = []
+    if nfull:
+        parts.append(q[:, :, : nfull * blk].reshape(B, H, nfull, blk, D).mean(dim=3))
+    if S % blk:
+        parts.append(q[:, :, nfull * blk:].mean(dim=2, keepdim=True))
+    qmean = torch.cat(parts, dim=2) * 1.0 / D ** 0.5
+    score = torch.einsum("bhmd,bhnd->bhmn", qmean, k)
     kv_indices = torch.topk(score, select_k, dim=-1, sorted=True).indices.to(torch.int32)
+    nb = (S + blk - 1) // blk
     return kv_indices, torch.full((B, H, nb), select_k, device=q.device, dtype=torch.int32)
 
 

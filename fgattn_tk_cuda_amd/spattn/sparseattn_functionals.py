@@ -42,10 +42,21 @@ def baseline_attn_maxq_denom(query, key, value, current_layer=None, ditrun=None,
     return _dense_with_stats(query, key, value)[0]
 
 
-def _sparse(query, key, value, kv_indices, kv_num_indices):
+def _sparse(query, key, value, kv_indices, kv_num_indices, order=None, cached=False):
+    """order: the work order that a cache computed when it stored these lists.  With it, or with
+    cached=True and no order (lists of even length), the step is one launch and allocates only
+    the output; without, ``sp_attn`` derives the order from the counts on every call."""
     out = _out_like(query)
-    spattn_interface.sp_attn(out, *_c(query, key, value, kv_indices, kv_num_indices))
+    if order is not None or cached:
+        spattn_interface.sp_attn_ex(out, None, *_c(query, key, value, kv_indices, kv_num_indices), order, 0.0, 0)
+    else:
+        spattn_interface.sp_attn(out, *_c(query, key, value, kv_indices, kv_num_indices))
     return out
+
+
+def _cached_order(mask_cache, layer):
+    get = getattr(mask_cache, "get_order", None)
+    return get(layer) if get is not None else None
 
 
 def attn_computed_with_sparse_mask_python(query, key, value, current_layer=None, ditrun=None, *args, **kwargs):
@@ -79,7 +90,7 @@ def compute_cache_and_attn_cuda(query, key, value, *args, **kwargs):
 def sparse_attn_from_cache_cuda(query, key, value, *args, **kwargs):
     """Sparse attention from cached lists (:88-93)."""
     kv_indices, kv_num_indices = kwargs["mask_cache"].get_mask_from_cache(kwargs.get("current_layer"))
-    return _sparse(query, key, value, kv_indices, kv_num_indices)
+    return _sparse(query, key, value, kv_indices, kv_num_indices, _cached_order(kwargs["mask_cache"], kwargs.get("current_layer")))
 
 
 def cached_attn_cuda(query, key, value, current_layer, ditrun, *args, **kwargs):
@@ -93,7 +104,27 @@ def cached_attn_cuda(query, key, value, current_layer, ditrun, *args, **kwargs):
         mask_cache.update_cache(current_layer, kv_indices, kv_num_indices)
         return out
     kv_indices, kv_num_indices = mask_cache.get_mask_from_cache(current_layer)
-    return _sparse(query, key, value, kv_indices, kv_num_indices)
+    return _sparse(query, key, value, kv_indices, kv_num_indices, _cached_order(mask_cache, current_layer))
+
+
+def blockcached_attn_cuda(query, key, value, current_layer, ditrun, *args, **kwargs):
+    """cached_attn_cuda at the granularity of 64-key blocks (no counterpart in the reference):
+    on the refresh steps dense attention with statistics, then the bit-packed threshold sweep and
+    the block lists for q-blocks of ``qblk`` rows (64 or 128, default 128), kept in a
+    ``mask_utils.BlockListCache``; on every other step ``sp_attn_block`` over the cached lists in
+    their cached work order - one launch."""
+    mask_cache = kwargs["mask_cache"]
+    qblk = kwargs.get("qblk", 128)
+    if mask_cache.run_fullattn(ditrun):
+        out, max_q, denom = _dense_with_stats(query, key, value)
+        blk_idx, blk_cnt = mask_utils.qk_blocklists_from_maxq_denom_cuda(max_q, denom, query, key, kwargs["thresh"], qblk)
+        mask_cache.update_cache(current_layer, blk_idx, blk_cnt)
+        return out
+    blk_idx, blk_cnt = mask_cache.get_mask_from_cache(current_layer)
+    out = _out_like(query)
+    spattn_interface.sp_attn_block(out, None, *_c(query, key, value, blk_idx, blk_cnt), mask_cache.get_order(current_layer),
+                                   qblk, 0.0, 0)
+    return out
 
 
 def bitmaskcached_attn_cuda(query, key, value, current_layer, ditrun, *args, **kwargs):

@@ -21,6 +21,11 @@ pinned (none of them is "parity unpinned"):
 * ``booleanmask_to_indexmask`` - integer exact; ``np.flatnonzero`` per row and
   a pure-Python loop on small inputs.
 * ``all_index_mask``           - ``arange`` closed form (include/utils.cuh:73-93).
+* ``booleanmask_rows``          - for 128-row q-blocks it is ``booleanmask_128 > 0``; for 64-row
+  q-blocks the OR of its two halves is the 128-row mask, and it equals max-pooling a
+  thresholded torch softmax over 64 rows.
+* ``block_mask_from_votes`` / ``block_lists_from_mask`` - integer exact; pure-Python loops over
+  every (row, block, key) on small inputs, ragged last block and keys >= seq included.
 * ``pack_mask`` / ``unpack_mask`` / ``packedmask_to_indexmask`` - ``numpy.packbits`` and round trips.
 * ``qblock_mean_scores``       - the reference's own torch expressions
   (python/spattn/mask_utils.py:390-410) evaluated in bf16 on the CPU.
@@ -281,6 +286,60 @@ def block_mask_from_votes(votes, seq: int, kvblk: int = 64):
     if pad:
         m = np.concatenate([m, np.zeros((B, H, SB, pad), bool)], axis=-1)
     return m.reshape(B, H, SB, nb, kvblk).any(axis=-1)
+
+
+def booleanmask_rows(max_q, denom, q, k, thresh: float, *, qblk: int = 128, kv_len: int | None = None,
+                     scale: float | None = None):
+    """The `> 0` view of the threshold mask for q-blocks of qblk rows (64 or 128):
+    M[I,c] = max_{r in I} p[r,c] > thresh with p as in ``booleanmask_128``
+    (include/mask_utils.cuh:231-238; a q-block votes if one of its 16-row groups does, and the
+    groups of a 64-row q-block are four of the eight of its 128-row block).
+    Returns (mask bool [B,H,ceil(S/qblk),kv_len], pmax fp32 of the same shape)."""
+    q = np.asarray(q, np.float32)
+    k = np.asarray(k, np.float32)
+    B, H, S, D = q.shape
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    kv = S if kv_len is None else kv_len
+    nq = ceil_div(S, qblk)
+    mx = np.asarray(max_q, np.float32).reshape(B, H, -1)
+    dn = np.asarray(denom, np.float32).reshape(B, H, -1)
+    pmax = np.zeros((B, H, nq, kv), np.float32)
+    for b in range(B):
+        for h in range(H):
+            for i in range(nq):
+                r0, r1 = i * qblk, min(S, (i + 1) * qblk)
+                s = q[b, h, r0:r1] @ k[b, h, :kv].T
+                p = np.exp2((s - mx[b, h, r0:r1, None]) * np.float32(LOG2E * scale)) / dn[b, h, r0:r1, None]
+                pmax[b, h, i] = p.astype(np.float32).max(axis=0)
+    return pmax > np.float32(thresh), pmax
+
+
+def block_lists_from_mask(mask, seq: int, *, kvblk: int = 64, max_blocks: int | None = None, fill: int = -1):
+    """Key mask -> ascending lists of kept key blocks: block J is kept when a key c in
+    [kvblk*J, kvblk*J + kvblk) with c < seq is set (mask > 0).  The block form of
+    ``booleanmask_to_indexmask`` (include/mask_utils.cuh:292-300 per key).
+    Returns (blk_idx int32 [B,H,SB,max_blocks] with `fill` behind the kept ids,
+    blk_cnt int32 [B,H,SB], blockmask bool [B,H,SB,ceil(mask_stride/kvblk)])."""
+    m = np.asarray(mask)
+    B, H, SB, MS = m.shape
+    nb = ceil_div(MS, kvblk)
+    bm = np.zeros((B, H, SB, nb), bool)
+    lim = min(seq, MS)
+    live = block_mask_from_votes(m, lim, kvblk) if lim > 0 else np.zeros((B, H, SB, 0), bool)
+    bm[..., : live.shape[-1]] = live
+    if max_blocks is None:
+        max_blocks = nb
+    idx = np.full((B, H, SB, max_blocks), fill, np.int32)
+    cnt = np.zeros((B, H, SB), np.int32)
+    for b in range(B):
+        for h in range(H):
+            for i in range(SB):
+                nz = np.flatnonzero(bm[b, h, i])
+                cnt[b, h, i] = nz.size
+                w = min(nz.size, max_blocks)
+                idx[b, h, i, :w] = nz[:w]
+    return idx, cnt, bm
 
 
 def pack_mask(mask):

@@ -252,6 +252,77 @@ def test_cfg4_padded_threshold_pipeline(dev):
         near = np.abs(pmax - thr) <= 1e-2 * thr
         assert np.array_equal((mh[0, h, i, :S] > 0) | near, (pmax > thr) | near), "mask row (%d,%d)" % (h, i)
     del mh
+    # block route: the sweep with bit outputs equals the packed vote mask; block lists from the bits
+    # and from the votes agree with each other and with the plain loop over the device's mask
+    pk128 = torch.full_like(packed, 0xA5)
+    capi.booleanmask_packed(pk128, mx, dn, qd, kd, thr, qblk=128)
+    assert torch.equal(pk128, packed)
+    nb = Sp // 64
+    bi = torch.full((B, H, SB, nb), -1, dtype=torch.int32, device=dev)
+    bc = torch.zeros((B, H, SB), dtype=torch.int32, device=dev)
+    bm = torch.empty((B, H, SB, nb), dtype=torch.uint8, device=dev)
+    capi.packedmask_to_blocklists(bi, bc, pk128, S, blockmask=bm)
+    bi2 = torch.full_like(bi, -1)
+    bc2 = torch.zeros_like(bc)
+    capi.booleanmask_to_blocklists(bi2, bc2, mask, S)
+    assert torch.equal(bi, bi2) and torch.equal(bc, bc2)
+    assert torch.equal(bm.bool(), blockmask)
+    assert torch.equal(bc, blockmask.sum(-1).int())
+    ar = torch.arange(nb, device=dev, dtype=torch.int32)
+    want_bi = torch.where(blockmask, ar, torch.full_like(ar, 1 << 20)).sort(-1).values
+    want_bi = torch.where(want_bi == (1 << 20), torch.full_like(want_bi, -1), want_bi)
+    assert torch.equal(bi, want_bi)
+    # 64-row q-blocks: two bit rows per 128-row block that OR to it; block lists of 12288 rows
+    n64 = orc.ceil_div(S, 64)
+    pk64 = torch.full((B, H, n64, Sp // 8), 0xA5, dtype=torch.uint8, device=dev)
+    capi.booleanmask_packed(pk64, mx, dn, qd, kd, thr, qblk=64)
+    assert torch.equal(pk64[:, :, 0::2] | pk64[:, :, 1::2], packed)
+    bi64 = torch.full((B, H, n64, nb), -1, dtype=torch.int32, device=dev)
+    bc64 = torch.zeros((B, H, n64), dtype=torch.int32, device=dev)
+    capi.packedmask_to_blocklists(bi64, bc64, pk64, S)
+    dens64 = float(bc64.float().mean()) / orc.ceil_div(S, 64)
+    assert 0.03 < dens64 < dens, (dens64, dens)
+    bits64 = pk64.cpu().numpy()
+    for h, i in blocks:
+        for half in (0, 1):
+            r = slice(i * 128 + 64 * half, min(S, i * 128 + 64 * half + 64))
+            if r.start >= S:
+                continue
+            s = f32(q[0, h, r]) @ kf[0, h].T
+            p = np.exp2((s - f32(mx)[0, h, 0, r, None]) * (orc.LOG2E / 8.0)) / f32(dn)[0, h, 0, r, None]
+            pmax = p.max(0)
+            near = np.abs(pmax - thr) <= 1e-2 * thr
+            got = np.unpackbits(bits64[0, h, 2 * i + half], bitorder="little")[:S].astype(bool)
+            assert np.array_equal(got | near, (pmax > thr) | near), "64-row bits (%d,%d,%d)" % (h, i, half)
+            lst = bi64[0, h, 2 * i + half, : int(bc64[0, h, 2 * i + half])].cpu().numpy()
+            assert np.array_equal(lst, np.flatnonzero(np.pad(got, (0, nb * 64 - S)).reshape(nb, 64).any(1)))
+    del pk64, bits64, pk128, packed, mask
+    ob = torch.full_like(qd, float("nan"))
+    capi.sp_attn_blocks(ob, qd, kd, vd, bi, bc, qblk=128)
+    ob64 = torch.full_like(qd, float("nan"))
+    capi.sp_attn_blocks(ob64, qd, kd, vd, bi64, bc64, qblk=64)
+    assert torch.isfinite(ob.float()).all() and torch.isfinite(ob64.float()).all()
+    vf = f32(v)
+    bih, bch, bi64h, bc64h = bi.cpu().numpy(), bc.cpu().numpy(), bi64.cpu().numpy(), bc64.cpu().numpy()
+    for h, i in blocks:
+        r = slice(i * 128, min(S, (i + 1) * 128))
+        tok, num = orc.block_list_to_token_list(bih[:, h:h + 1, i:i + 1], bch[:, h:h + 1, i:i + 1], S)
+        lst = tok[0, 0, 0, : num[0, 0, 0]]
+        pp, den, _ = orc._softmax_rows(f32(q[0, h, r]) @ kf[0, h, lst].T, 0.125, True)
+        assert_close_o(f32(ob[0, h, r]), (pp @ vf[0, h, lst]) / den[:, None], "cfg4 block rows (%d,%d)" % (h, i))
+        for half in (0, 1):
+            r = slice(i * 128 + 64 * half, min(S, i * 128 + 64 * half + 64))
+            if r.start >= S:
+                continue
+            j = 2 * i + half
+            tok, num = orc.block_list_to_token_list(bi64h[:, h:h + 1, j:j + 1], bc64h[:, h:h + 1, j:j + 1], S)
+            lst = tok[0, 0, 0, : num[0, 0, 0]]
+            if lst.size == 0:          # a q-block without a key: zeros
+                assert not f32(ob64[0, h, r]).any()
+                continue
+            pp, den, _ = orc._softmax_rows(f32(q[0, h, r]) @ kf[0, h, lst].T, 0.125, True)
+            assert_close_o(f32(ob64[0, h, r]), (pp @ vf[0, h, lst]) / den[:, None], "cfg4 block rows q64 (%d,%d)" % (h, j))
+    del ob, ob64
     o = torch.full_like(qd, float("nan"))
     capi.sp_attn(o, qd, kd, vd, kvi, kvn)
     assert torch.isfinite(o.float()).all()

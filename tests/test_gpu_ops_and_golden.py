@@ -122,6 +122,112 @@ def test_operator_extension_on_device(dev):
         ops.sp_attn(o, q, k, v, kvi[:, :, :3].contiguous(), kvn)
 
 
+def test_extended_operators_on_device(dev):
+    """The operators beyond the reference's seven: kv length, scale and lse through torch.ops, the
+    block-list attention, the bit-packed sweep, the block lists, the reusable work order.  Each
+    against the oracle or, where an operator restates another, bit for bit against that one."""
+    print("case extended torch ops", flush=True)
+    import fgattn_tk_cuda_amd.spattn.cuda_attn  # noqa: F401
+    from fgattn_tk_cuda_amd.spattn import mask_utils as mu
+
+    ops = torch.ops.cuda_attn
+    B, H, S, D = 1, 2, 1000, 64
+    kv = 870
+    q, k, v = to_dev(dev, *wl.clustered_qkv(B, H, S, D, seed=73, sigma=0.6))
+    scale = 0.1
+    # full_attn_ex: kv length + scale + lse against torch on the cut keys
+    want = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float()[:, :, :kv], v.float()[:, :, :kv], scale=scale)
+    wlse = torch.logsumexp(torch.einsum("bhsd,bhtd->bhst", q.float(), k.float()[:, :, :kv]) * scale, -1)
+    o = torch.full_like(q, float("nan"))
+    lse = torch.full((B, H, S), float("nan"), device=dev)
+    ops.full_attn_ex(o, lse, q, k, v, scale, kv)
+    assert_close_o(f32(o), f32(want), "full_attn_ex")
+    assert_close_stat(f32(lse), f32(wlse), "full_attn_ex lse")
+    o0 = torch.full_like(q, float("nan"))
+    ops.full_attn_ex(o0, None, q, k, v, 0.0, 0)
+    o1 = torch.full_like(q, float("nan"))
+    ops.full_attn(o1, q, k, v)
+    assert torch.equal(o0, o1)
+    # statistics with a kv length, then the vote mask and the bit-packed sweep with it
+    Sp, SB = 1024, 8
+    mx = torch.empty((B, H, 1, Sp), device=dev)
+    dn = torch.empty((B, H, 1, Sp), device=dev)
+    ops.maxq_denom_ex(mx, dn, q, k, 0.0, kv)
+    wmx, wdn = orc.maxq_denom(f32(q), f32(k), kv_len=kv)
+    assert_close_stat(f32(mx)[..., :S], wmx[..., :S], "maxq_denom_ex max", atol=1e-3)
+    assert_close_stat(f32(dn)[..., :S], wdn[..., :S], "maxq_denom_ex denom")
+    o2 = torch.full_like(q, float("nan"))
+    mx2, dn2 = torch.empty_like(mx), torch.empty_like(dn)
+    ops.fullattn_maxq_denom_ex(o2, mx2, dn2, q, k, v, 0.0, kv)
+    wo2 = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float()[:, :, :kv], v.float()[:, :, :kv])
+    assert_close_o(f32(o2), f32(wo2), "fullattn_maxq_denom_ex")
+    assert_close_stat(f32(dn2), f32(dn), "fused denom with kv_len")
+    thr = 0.02
+    votes = torch.zeros((B, H, SB, Sp), dtype=torch.int32, device=dev)
+    ops.booleanmask_128_ex(votes, mx, dn, q, k, thr, 0.0, kv)
+    assert not bool(votes[..., kv:].any()) and bool(votes.any())
+    for qblk in (128, 64):
+        nq = (S + qblk - 1) // qblk
+        packed = torch.full((B, H, nq, Sp // 8), 0xA5, dtype=torch.uint8, device=dev)
+        ops.booleanmask_packed(packed, mx, dn, q, k, thr, qblk, 0.0, kv)
+        if qblk == 128:
+            assert torch.equal(packed, mu.pack(votes > 0))
+        else:
+            assert torch.equal(packed[:, :, 0::2] | packed[:, :, 1::2], mu.pack(votes > 0))
+        assert torch.equal(packed, mu.qk_packedmask_from_maxq_denom_cuda(mx, dn, q, k, thr, qblk, kv))
+        # block lists: operator == oracle on the device's own bits; packed and votes sources agree
+        blk_idx, blk_cnt, bm = mu.packedmask_to_blocklists_cuda(packed, kv, with_blockmask=True)
+        wi, wn, wbm = orc.block_lists_from_mask(orc.unpack_mask(packed.cpu().numpy()), kv, fill=-1)
+        assert np.array_equal(blk_idx.cpu().numpy(), wi) and np.array_equal(blk_cnt.cpu().numpy(), wn)
+        assert np.array_equal(bm.cpu().numpy(), wbm.astype(np.uint8))
+        if qblk == 128:
+            bi2, bc2 = mu.bitmask_to_blocklists_cuda(votes, kv)
+            assert torch.equal(bi2, blk_idx) and torch.equal(bc2, blk_cnt)
+        # sp_attn_block with lse, scale, kv length and a work order
+        order = mu.qblock_order_cuda(blk_cnt)
+        assert np.array_equal(order.cpu().numpy(), orc.qblock_order(wn))
+        ob = torch.full_like(q, float("nan"))
+        lb = torch.full((B, H, S), float("nan"), device=dev)
+        ops.sp_attn_block(ob, lb, q, k, v, blk_idx, blk_cnt, order, qblk, scale, kv)
+        tok, num = orc.block_list_to_token_list(wi, wn, kv, mask_stride=Sp)
+        wo, wl_ = orc.sp_attn(f32(q), f32(k), f32(v), tok, num, qblk=qblk, scale=scale)
+        assert_close_o(f32(ob), wo, "sp_attn_block q%d" % qblk)
+        assert_close_stat(f32(lb), wl_, "sp_attn_block lse q%d" % qblk)
+        ob2 = torch.full_like(q, float("nan"))
+        ops.sp_attn_block(ob2, None, q, k, v, blk_idx, blk_cnt, None, 0, scale, kv)     # no order, inferred q-block
+        assert torch.equal(ob, ob2)
+        # the same keys as token lists through sp_attn_ex: the operator's own cross-check
+        tk, nm = torch.from_numpy(tok).to(dev), torch.from_numpy(num).to(dev)
+        ot = torch.full_like(q, float("nan"))
+        lt = torch.full((B, H, S), float("nan"), device=dev)
+        ops.sp_attn_ex(ot, lt, q, k, v, tk, nm, mu.qblock_order_cuda(nm), scale, kv)
+        assert_close_o(f32(ot), wo, "sp_attn_ex q%d" % qblk)
+        assert_close_stat(f32(lt), wl_, "sp_attn_ex lse q%d" % qblk)
+    # sp_attn_ex without extras == sp_attn
+    kvi, kvn = mu.qk_indexmask_cuda(q, k, thr)
+    oa, ob_ = torch.full_like(q, float("nan")), torch.full_like(q, float("nan"))
+    ops.sp_attn(oa, q, k, v, kvi, kvn)
+    ops.sp_attn_ex(ob_, None, q, k, v, kvi, kvn, None, 0.0, 0)
+    assert torch.equal(oa, ob_)
+    # the pure-torch definition of the block lists against the device path (kv length = S here)
+    bi_d, bc_d = mu.qk_blocklists_cuda(q, k, thr, qblk=128)
+    bi_r, bc_r, _ = mu.qk_blocklists(q.float(), k.float(), thr, qblk=128)
+    mxs, dns = mu._stats_buffers(q)
+    ops.maxq_denom(mxs, dns, q, k)
+    _, pmax = orc.booleanmask_128(f32(mxs), f32(dns), f32(q), f32(k), thr)
+    if not (np.abs(pmax - thr) <= 1e-2 * thr).any():
+        assert torch.equal(bc_d, bc_r) and torch.equal(bi_d, bi_r)
+    else:
+        assert (bc_d - bc_r).abs().max().item() <= 2
+    # bad arguments raise
+    with pytest.raises(RuntimeError):
+        ops.full_attn_ex(o, None, q, k, v, 0.0, S + 1)
+    with pytest.raises(RuntimeError):
+        ops.sp_attn_block(o, None, q, k, v, blk_idx, blk_cnt, order[:3].contiguous(), 64, 0.0, 0)
+    with pytest.raises(RuntimeError):
+        ops.booleanmask_packed(packed, mx, dn, q, k, thr, 32, 0.0, 0)
+
+
 def test_functionals_with_mask_cache(dev):
     print("case functionals", flush=True)
     from fgattn_tk_cuda_amd.spattn import mask_utils as mu, sparseattn_functionals as fn
@@ -140,6 +246,18 @@ def test_functionals_with_mask_cache(dev):
         want, _ = orc.sp_attn(f32(q), f32(k), f32(v), kvi.cpu().numpy(), kvn.cpu().numpy(), qblk=128)
         assert_close_o(f32(o1), want, "sparse step from %s" % type(cache).__name__)
         assert 0 < kvn.float().mean().item() < S
+        if isinstance(cache, mu.NaiveMaskCache):
+            assert cache.get_order(7) is not None and cache.get_order(7).numel() == kvn.numel()
+    for qblk in (64, 128):
+        cache = mu.BlockListCache([0])
+        o0 = fn.blockcached_attn_cuda(q, k, v, 7, 0, thresh=0.01, qblk=qblk, mask_cache=cache)
+        assert_close_o(f32(o0), f32(dense), "block cache fill step")
+        o1 = fn.blockcached_attn_cuda(q, k, v, 7, 1, thresh=0.01, qblk=qblk, mask_cache=cache)
+        bi, bc = cache.get_mask_from_cache(7)
+        tok, num = orc.block_list_to_token_list(bi.cpu().numpy(), bc.cpu().numpy(), S)
+        wb, _ = orc.sp_attn(f32(q), f32(k), f32(v), tok, num, qblk=qblk)
+        assert_close_o(f32(o1), wb, "block sparse step q%d" % qblk)
+        assert 0 < bc.float().mean().item() < (S + 63) // 64
     o2 = fn.attn_computed_with_sparse_mask_cuda(q, k, v, thresh=0.01, blocksz=128)
     assert_close_o(f32(o2), want, "attn_computed_with_sparse_mask_cuda")
     o3 = fn.attn_2xmask_cuda(q, k, v, 0, 0, blocksz=128)

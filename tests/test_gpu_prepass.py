@@ -134,6 +134,128 @@ def test_bit_kernels_more_rows_than_one_round_of_the_grid(dev):
     assert np.array_equal(kvi.cpu().numpy(), wi)
 
 
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("S,kv_len", [(512, 0), (1000, 0), (1000, 870), (200, 0), (1090, 1000)])
+def test_booleanmask_packed_bits(dev, D, S, kv_len):
+    """The sweep with bit outputs.  128-row q-blocks: bit for bit the packed form of the int32 vote
+    mask of the same sweep.  64-row q-blocks: the two halves OR to the 128-row bits exactly, and
+    each half agrees with the oracle outside the threshold band.  Every word is written."""
+    print("case booleanmask packed", D, S, kv_len, flush=True)
+    B, H = 1, 3
+    q, k, v = wl.clustered_qkv(B, H, S, D, seed=43, sigma=0.7)
+    qd, kd = to_dev(dev, q, k)
+    kv = kv_len or S
+    Sp = orc.padded_len(S)
+    SB, n64 = Sp // 128, orc.ceil_div(S, 64)
+    mx = torch.empty((B, H, 1, Sp), device=dev)
+    dn = torch.empty((B, H, 1, Sp), device=dev)
+    capi.maxq_denom(mx, dn, qd, kd, kv_len=kv_len)
+    m64, p64 = orc.booleanmask_rows(f32(mx), f32(dn), f32(q), f32(k), 1.0, qblk=64, kv_len=kv)
+    thr = float(np.quantile(p64, 0.75))
+    mask = torch.full((B, H, SB, Sp), -7, dtype=torch.int32, device=dev)
+    capi.booleanmask_128(mask, mx, dn, qd, kd, thr, kv_len=kv_len)
+    want128 = orc.pack_mask(mask.cpu().numpy())
+    p128 = torch.full((B, H, SB, Sp // 8), 0xA5, dtype=torch.uint8, device=dev)
+    capi.booleanmask_packed(p128, mx, dn, qd, kd, thr, qblk=128, kv_len=kv_len)
+    assert np.array_equal(p128.cpu().numpy(), want128)
+    pk64 = torch.full((B, H, n64, Sp // 8), 0xA5, dtype=torch.uint8, device=dev)
+    capi.booleanmask_packed(pk64, mx, dn, qd, kd, thr, qblk=64, kv_len=kv_len)
+    g64 = pk64.cpu().numpy()
+    both = np.zeros((B, H, 2 * SB, Sp // 8), np.uint8)
+    both[:, :, :n64] = g64
+    assert np.array_equal(both[:, :, 0::2] | both[:, :, 1::2], want128)
+    bits = orc.unpack_mask(g64)
+    assert not bits[..., kv:].any()
+    m64 = p64 > np.float32(thr)
+    near = np.abs(p64 - thr) <= BAND * thr
+    dis = (bits[..., :kv] != m64) & ~near
+    assert dis.sum() == 0, "%d mismatches outside the threshold band" % dis.sum()
+    assert 0.01 < m64.mean() < 0.9
+
+
+@pytest.mark.parametrize("SB,ms,seq,max_blocks,density", [
+    (3, 384, 300, 6, 0.1), (2, 2176, 2100, 34, 0.05), (5, 128, 128, 2, 0.5), (1, 4096, 1, 64, 1.0),
+    (2, 8192 + 256, 8192 + 200, 40, 0.08), (2, 1024, 0, 16, 0.5), (3, 4096, 4000, 64, 0.0), (2, 32768, 32760, 512, 0.02),
+    (1, 4096, 4096, 5, 0.3)])
+def test_block_lists_bit_exact(dev, SB, ms, seq, max_blocks, density):
+    """Key mask -> block mask -> ascending block lists, from the bit-packed mask and from the int32
+    votes: ids, counts, fill and the block mask bit for bit (incl. a list longer than max_blocks)."""
+    print("case block lists", SB, ms, seq, max_blocks, density, flush=True)
+    B, H = 2, 2
+    rng = np.random.default_rng(90)
+    mask = _run_mask(rng, (B, H, SB, ms), density) if density < 1.0 else np.ones((B, H, SB, ms), np.int32)
+    wi, wn, wbm = orc.block_lists_from_mask(mask, seq, max_blocks=max_blocks, fill=-3)
+    md = torch.from_numpy(mask).to(dev)
+    pk = torch.from_numpy(orc.pack_mask(mask)).to(dev)
+    for src in ("packed", "votes"):
+        bi = torch.full((B, H, SB, max_blocks), -3, dtype=torch.int32, device=dev)
+        bc = torch.full((B, H, SB), -1, dtype=torch.int32, device=dev)
+        bm = torch.full((B, H, SB, ms // 64), 7, dtype=torch.uint8, device=dev)
+        if src == "packed":
+            capi.packedmask_to_blocklists(bi, bc, pk, seq, blockmask=bm)
+        else:
+            capi.booleanmask_to_blocklists(bi, bc, md, seq, blockmask=bm)
+        assert np.array_equal(bc.cpu().numpy(), wn), src
+        assert np.array_equal(bi.cpu().numpy(), wi), src
+        assert np.array_equal(bm.cpu().numpy(), wbm.astype(np.uint8)), src
+        bi2 = torch.full((B, H, SB, max_blocks), -3, dtype=torch.int32, device=dev)
+        bc2 = torch.full((B, H, SB), -1, dtype=torch.int32, device=dev)
+        (capi.packedmask_to_blocklists if src == "packed" else capi.booleanmask_to_blocklists)(
+            bi2, bc2, pk if src == "packed" else md, seq)          # without the block mask output
+        assert torch.equal(bi, bi2) and torch.equal(bc, bc2)
+
+
+def test_block_lists_more_rows_than_one_round_of_the_grid(dev):
+    """8960 rows: both block-list kernels walk more rows than their grid holds waves."""
+    print("case block lists many rows", flush=True)
+    B, H, SB, ms, seq = 1, 70, 128, 256, 250
+    rng = np.random.default_rng(91)
+    mask = _run_mask(rng, (B, H, SB, ms), 0.1)
+    mask[0, 69, 127] = 2
+    wi, wn, _ = orc.block_lists_from_mask(mask, seq, fill=-1)
+    md = torch.from_numpy(mask).to(dev)
+    pk = torch.from_numpy(orc.pack_mask(mask)).to(dev)
+    for fn, src in ((capi.packedmask_to_blocklists, pk), (capi.booleanmask_to_blocklists, md)):
+        bi = torch.full((B, H, SB, ms // 64), -1, dtype=torch.int32, device=dev)
+        bc = torch.full((B, H, SB), -1, dtype=torch.int32, device=dev)
+        fn(bi, bc, src, seq)
+        assert np.array_equal(bc.cpu().numpy(), wn) and np.array_equal(bi.cpu().numpy(), wi)
+
+
+@pytest.mark.parametrize("qblk", [64, 128])
+@pytest.mark.parametrize("D,S", [(64, 1000), (128, 700)])
+def test_block_threshold_pipeline_feeds_block_attention(dev, qblk, D, S):
+    """maxq_denom -> bit-packed sweep -> block lists -> sp_attn_blocks: the block lists are those of
+    the device's own bits (exact), and the attention over them matches the oracle over the
+    expanded token lists."""
+    print("case block pipeline", qblk, D, S, flush=True)
+    B, H = 1, 2
+    q, k, v = wl.clustered_qkv(B, H, S, D, seed=63, sigma=0.7)
+    qd, kd, vd = to_dev(dev, q, k, v)
+    Sp = orc.padded_len(S)
+    nq = orc.ceil_div(S, qblk)
+    mx = torch.empty((B, H, 1, Sp), device=dev)
+    dn = torch.empty((B, H, 1, Sp), device=dev)
+    capi.maxq_denom(mx, dn, qd, kd)
+    pk = torch.empty((B, H, nq, Sp // 8), dtype=torch.uint8, device=dev)
+    capi.booleanmask_packed(pk, mx, dn, qd, kd, 0.03, qblk=qblk)
+    nb = Sp // 64
+    bi = torch.full((B, H, nq, nb), -1, dtype=torch.int32, device=dev)
+    bc = torch.zeros((B, H, nq), dtype=torch.int32, device=dev)
+    capi.packedmask_to_blocklists(bi, bc, pk, S)
+    wi, wn, _ = orc.block_lists_from_mask(orc.unpack_mask(pk.cpu().numpy()), S, fill=-1)
+    assert np.array_equal(bi.cpu().numpy(), wi) and np.array_equal(bc.cpu().numpy(), wn)
+    assert 0 < wn.mean() < nb
+    o = torch.full_like(qd, float("nan"))
+    lse = torch.empty((B, H, S), device=dev)
+    capi.sp_attn_blocks(o, qd, kd, vd, bi, bc, lse=lse, qblk=qblk)
+    tok, num = orc.block_list_to_token_list(wi, wn, S)
+    want, wlse = orc.sp_attn(f32(q), f32(k), f32(v), tok, num, qblk=qblk)
+    from helpers import assert_close_o, assert_close_stat
+    assert_close_o(f32(o), want, "block pipeline O")
+    assert_close_stat(f32(lse), wlse, "block pipeline lse")
+
+
 def test_all_index_mask(dev):
     print("case all_index_mask", flush=True)
     B, H, SB, S, ms = 2, 3, 5, 600, 640

@@ -106,3 +106,53 @@ def test_operator_extension_registers_the_seven_ops():
     torch.ops.cuda_attn.sp_attn(q, q, q, q, idx, idx)
     schema = str(torch.ops.cuda_attn.sp_attn.default._schema)
     assert "Tensor(a!) o" in schema and "kv_num_indices" in schema
+    # the seven reference schemas, character for character (python/extension.cpp:82,113,166,215,259,309,349)
+    ref = {
+        "full_attn": "cuda_attn::full_attn(Tensor(a!) o, Tensor q, Tensor k, Tensor v) -> ()",
+        "all_index_mask": "cuda_attn::all_index_mask(Tensor(a!) kv_indices, Tensor(b!) kv_num_indices, int batch, int heads, int seqblocks, int seq) -> ()",
+        "sp_attn": "cuda_attn::sp_attn(Tensor(a!) o, Tensor q, Tensor k, Tensor v, Tensor kv_indices, Tensor kv_num_indices) -> ()",
+        "fullattn_maxq_denom": "cuda_attn::fullattn_maxq_denom(Tensor(a!) o, Tensor(b!) o_max_q, Tensor(c!) o_denom, Tensor q, Tensor k, Tensor v) -> ()",
+        "maxq_denom": "cuda_attn::maxq_denom(Tensor(a!) o_max_q, Tensor(b!) o_denom, Tensor q, Tensor k) -> ()",
+        "booleanmask_128": "cuda_attn::booleanmask_128(Tensor(a!) booleanmask, Tensor o_max_q, Tensor o_denom, Tensor q, Tensor k, float threshold) -> ()",
+        "booleanmask_to_indexmask": "cuda_attn::booleanmask_to_indexmask(Tensor(a!) kv_indices, Tensor(b!) kv_numindices, Tensor booleanmask, int seq) -> ()",
+    }
+    for n, want in ref.items():
+        assert str(getattr(torch.ops.cuda_attn, n).default._schema) == want
+
+
+def test_extended_operators_are_registered_with_meta_kernels():
+    import fgattn_tk_cuda_amd.spattn.cuda_attn as ext
+
+    names = ["full_attn_ex", "sp_attn_ex", "sp_attn_block", "fullattn_maxq_denom_ex", "maxq_denom_ex", "booleanmask_128_ex",
+             "booleanmask_packed", "packedmask_to_blocklists", "booleanmask_to_blocklists", "qblock_order"]
+    for n in names:
+        assert hasattr(ext, n) and hasattr(torch.ops.cuda_attn, n)
+    q = torch.zeros((1, 2, 256, 128), dtype=torch.bfloat16, device="meta")
+    i4 = torch.zeros((1, 2, 4, 8), dtype=torch.int32, device="meta")
+    i3 = torch.zeros((1, 2, 4), dtype=torch.int32, device="meta")
+    lse = torch.zeros((1, 2, 256), device="meta")
+    torch.ops.cuda_attn.sp_attn_block(q, lse, q, q, q, i4, i3, None, 64, 0.0, 0)
+    torch.ops.cuda_attn.sp_attn_block(q, None, q, q, q, i4, i3, i3.reshape(-1), 64, 0.0, 0)
+    torch.ops.cuda_attn.full_attn_ex(q, None, q, q, q, 0.0, 100)
+    pk = torch.zeros((1, 2, 4, 32), dtype=torch.uint8, device="meta")
+    torch.ops.cuda_attn.packedmask_to_blocklists(i4, i3, None, pk, 256)
+    assert "Tensor(b!)? lse" in str(torch.ops.cuda_attn.sp_attn_block.default._schema)
+
+
+def test_topk_mask_definition_takes_the_reference_signature():
+    """(q, k, select_k, B, H, S, D, BLOCKSZ) as the reference defines it, or blocksz= alone as its
+    caller passes it; computed in the dtype of q."""
+    from fgattn_tk_cuda_amd.spattn import mask_utils as mu
+
+    q, k, _ = wl.randn_qkv(1, 2, 300, 64, seed=3)
+    a_idx, a_num = mu.qk_topkmask_indices(q, k, 40, 1, 2, 300, 64, 128)
+    b_idx, b_num = mu.qk_topkmask_indices(q, k, 40, blocksz=128)
+    assert torch.equal(a_idx, b_idx) and torch.equal(a_num, b_num)
+    assert a_idx.shape == (1, 2, 3, 40) and a_idx.dtype == torch.int32 and int(a_num[0, 0, 0]) == 40
+    qm, sc = orc.qblock_mean_scores(q.float().numpy(), k.float().numpy(), 128)
+    want = orc.topk_select(sc, 40)
+    got = np.sort(a_idx.numpy(), axis=-1)
+    # same keys wherever the 40th and 41st scores differ (ties may go either way in torch.topk)
+    srt = np.sort(sc, axis=-1)
+    clear = srt[..., -40] != srt[..., -41]
+    assert clear.any() and np.array_equal(got[clear], want[clear])

@@ -195,6 +195,77 @@ def test_booleanmask_to_indexmask_exact():
     assert num2[0, 0, 0] == 0 and np.all(idx2 == 128)
 
 
+@pytest.mark.parametrize("S", [300, 330])
+def test_booleanmask_rows_is_the_maxpooled_threshold_at_64_and_128_rows(S):
+    """M[I,c] for 64-row q-blocks against torch softmax + max_pool over 64 rows; the two halves
+    of a 128-row block OR to the 128-row mask, which is `booleanmask_128 > 0` exactly."""
+    B, H, D = 1, 2, 64
+    q, k, _ = (t.float() for t in wl.clustered_qkv(B, H, S, D, seed=12, sigma=0.7))
+    mx, dn = orc.maxq_denom(q.numpy(), k.numpy())
+    thr = 0.02
+    m128, p128 = orc.booleanmask_rows(mx, dn, q.numpy(), k.numpy(), thr, qblk=128)
+    m64, p64 = orc.booleanmask_rows(mx, dn, q.numpy(), k.numpy(), thr, qblk=64)
+    votes, pmax = orc.booleanmask_128(mx, dn, q.numpy(), k.numpy(), thr)
+    assert np.array_equal(m128, votes[..., :S] > 0) and np.array_equal(p128, pmax)
+    n64, n128 = orc.ceil_div(S, 64), orc.ceil_div(S, 128)
+    assert m64.shape == (B, H, n64, S) and m128.shape == (B, H, n128, S)
+    both = np.zeros((B, H, 2 * n128, S), bool)
+    both[:, :, :n64] = m64
+    assert np.array_equal(both[:, :, 0::2] | both[:, :, 1::2], m128)
+    for h in range(H):
+        p = torch.softmax(q[0, h] @ k[0, h].T / math.sqrt(D), -1)
+        hit = (p > thr).float()[None]
+        pooled = torch.nn.functional.max_pool2d(torch.nn.functional.pad(hit, (0, 0, 0, (-S) % 64)), (64, 1))[0] > 0
+        near = np.abs(p64[0, h] - thr) <= 1e-3 * thr
+        assert np.array_equal(m64[0, h] | near, pooled.numpy() | near)
+    # a short kv length cuts columns, nothing else
+    mk, _ = orc.booleanmask_rows(*orc.maxq_denom(q.numpy(), k.numpy(), kv_len=200), q.numpy(), k.numpy(), thr, qblk=64, kv_len=200)
+    assert mk.shape[-1] == 200
+
+
+def test_block_mask_and_block_lists_by_brute_force():
+    """MB[I,J] = OR of the keys of block J below seq; lists = ascending kept block ids, fill behind
+    them, exact counts - against plain loops, with a ragged last block, set keys at and past seq,
+    an empty row, a full row and a list cut off at max_blocks."""
+    rng = np.random.default_rng(13)
+    B, H, SB, MS, seq = 1, 2, 4, 384, 300
+    mask = ((rng.random((B, H, SB, MS)) < 0.03) * rng.integers(1, 9, (B, H, SB, MS))).astype(np.int32)
+    mask[0, 0, 0] = 0
+    mask[0, 0, 1] = 3
+    mask[0, 1, 2, :] = 0
+    mask[0, 1, 2, 299] = 1          # the last key below seq: block 4 (keys 256..319) is kept
+    mask[0, 1, 2, 300] = 1          # at seq: ignored
+    mask[0, 1, 3, :] = 0
+    mask[0, 1, 3, 320:] = 1         # only keys past seq: nothing is kept
+    bm = orc.block_mask_from_votes(mask, seq)
+    nb = orc.ceil_div(seq, 64)
+    assert bm.shape == (B, H, SB, nb)
+    for h in range(H):
+        for i in range(SB):
+            for J in range(nb):
+                want = any(mask[0, h, i, c] > 0 for c in range(64 * J, min(64 * J + 64, seq)))
+                assert bm[0, h, i, J] == want, (h, i, J)
+    idx, cnt, full = orc.block_lists_from_mask(mask, seq, fill=-5)
+    assert full.shape == (B, H, SB, MS // 64) and np.array_equal(full[..., :nb], bm) and not full[..., nb:].any()
+    for h in range(H):
+        for i in range(SB):
+            kept = [J for J in range(nb) if bm[0, h, i, J]]
+            assert cnt[0, h, i] == len(kept) and idx[0, h, i, : len(kept)].tolist() == kept
+            assert np.all(idx[0, h, i, len(kept):] == -5)
+    assert cnt[0, 0, 0] == 0 and cnt[0, 0, 1] == nb and idx[0, 1, 2, :1].tolist() == [4] and cnt[0, 1, 2] == 1 and cnt[0, 1, 3] == 0
+    idx2, cnt2, _ = orc.block_lists_from_mask(mask, seq, max_blocks=2, fill=-5)
+    assert np.array_equal(cnt2, cnt) and np.array_equal(idx2, idx[..., :2])
+    # a bool mask and the packed form of the same mask give the same blocks
+    assert np.array_equal(orc.block_mask_from_votes(orc.unpack_mask(orc.pack_mask(mask)), seq), bm)
+    # block lists are the token lists of the reference restricted to aligned runs: expanding them
+    # covers every kept key
+    tok, num = orc.block_list_to_token_list(idx, cnt, seq, mask_stride=MS)
+    ki, kn = orc.booleanmask_to_indexmask(mask, seq)
+    for h in range(H):
+        for i in range(SB):
+            assert set(ki[0, h, i, : kn[0, h, i]]) <= set(tok[0, h, i, : num[0, h, i]])
+
+
 def test_all_index_mask():
     idx, num = orc.all_index_mask(1, 2, 3, 300, 384)
     assert idx.shape == (1, 2, 3, 384) and np.all(idx == np.arange(384)) and np.all(num == 300)
