@@ -31,12 +31,18 @@ from fgattn_tk_cuda_amd import capi, workloads as wl  # noqa: E402
 PEAK_BF16_TFLOPS = 2500.0
 PEAK_HBM_GBPS = 8000.0
 
-# HBM-side bytes per launch from `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs of this
-# file (--only sparse / --only compact), scaled by what the same counters read for the plain
-# 1 GiB copy of --only copy (FETCH_SIZE x2.0, WRITE_SIZE x1.0).  Text summaries of those runs
-# sit in profiles/counters_*.txt; they are measured offline, not in this process.
-TRAFFIC_SPARSE_BYTES = 4.746e9 + 0.2726e9   # rocprofv3 FETCH_SIZE x2.0 + WRITE_SIZE x1.0, see profiles/
-TRAFFIC_COMPACT_BYTES = 805.4e6 + 64.5e6    # fetch + write of compact_kernel
+# HBM-side bytes per launch come from `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs of
+# this file (--only sparse / --only compact), scaled by what the same counters read for the plain
+# 1 GiB copy of --only copy.  They are measured offline, not in this process: the figures, the
+# scale factors and the commands sit in profiles/traffic.json next to the counter summaries, and a
+# kernel without an entry there reports null.
+def measured_traffic(key):
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            e = json.load(f)["kernels"][key]
+        return float(e["fetch_bytes"]) + float(e["write_bytes"])
+    except (OSError, KeyError, ValueError):
+        return None
 
 
 # The part raises its clocks over the first tens of milliseconds of sustained load: the same
@@ -106,13 +112,17 @@ def bench_tokens(dev, steps, warmup, seed=0, res=None):
     return dict(ms=ms, flops=res["flops"], list_bytes=4.0 * tok.numel())
 
 
-def bench_zipf(dev, steps, warmup, seed=0):
+def bench_zipf(dev, steps, warmup, seed=0, hi=None):
     """cfg5: B=1 H=8 N=65536 d=128, 128-row q-blocks, per-row block counts ~ Zipf(1.2) clipped to
-    [1,1024]: the default schedule against the longest-list-first work order (same results)."""
+    [1,hi] (default 1024): the default schedule against the longest-list-first work order (same
+    results).  Clipped at 1024 the counts have a mean of about 28 % of the 1024 key blocks and a
+    fifth of the rows sit at the clip; clipped at 64 the mean is the 3 % the workload's
+    description states."""
     c = wl.CONFIGS["cfg5_zipf_64k"]
     B, H, S, D, qblk = c["B"], c["H"], c["S"], c["D"], c["qblk"]
+    hi = hi or c["max_blocks"]
     q, k, v = (t.to(dev) for t in wl.randn_qkv(B, H, S, D, seed=seed))
-    cnt = wl.zipf_counts(B, H, S // qblk, s=c["zipf_s"], lo=1, hi=c["max_blocks"], seed=seed + 3)
+    cnt = wl.zipf_counts(B, H, S // qblk, s=c["zipf_s"], lo=1, hi=hi, seed=seed + 3)
     bi, bc = (t.to(dev) for t in wl.ragged_block_lists(B, H, S, qblk, 64, cnt, seed=seed + 4))
     o = torch.empty_like(q)
     order = torch.empty((bc.numel(),), dtype=torch.int32, device=dev)
@@ -125,19 +135,35 @@ def bench_zipf(dev, steps, warmup, seed=0):
         capi.sp_attn_blocks(o, q, k, v, bi, bc, qblk=qblk, order=order)
 
     ms1, _ = time_steps(ordered, steps, warmup)
-    return dict(ms_default=ms0, ms_ordered=ms1, ms_order_kernel=ms_o, flops=flops, kept_blocks=int(cnt.sum()))
+    return dict(ms_default=ms0, ms_ordered=ms1, ms_order_kernel=ms_o, flops=flops, kept_blocks=int(cnt.sum()),
+                mean_blocks=float(cnt.mean()), density=float(cnt.mean()) / (S // 64), saturated_rows=float((cnt == hi).mean()),
+                clip=hi)
 
 
-def bench_compaction(dev, steps, warmup, seed=0):
+def bench_zipf_sparse(dev, steps, warmup, seed=0):
+    return bench_zipf(dev, steps, warmup, seed=seed, hi=64)
+
+
+def _iid_mask(dev, seed):
+    c = wl.CONFIGS["cfg4_threshold_padded"]
+    B, H, S = c["B"], c["H"], c["S"]
+    ms_ = 128 * wl.ceil_div(S, 128)
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    return (torch.rand((B, H, ms_ // 128, ms_), device=dev, generator=g) < c["keep"]).to(torch.int32)
+
+
+def bench_compaction(dev, steps, warmup, seed=0, mask=None):
     """booleanmask_to_indexmask at the padded threshold workload: B=1, H=24, N=32760 -> mask
-    [1,24,256,32768] int32 with ~8 % of the entries set."""
+    [1,24,256,32768] int32.  mask: the vote mask of the threshold sweep (kept keys come in runs);
+    without one, an iid mask with 8 % of the entries set.  The counts are checked against the
+    mask's own row sums."""
     c = wl.CONFIGS["cfg4_threshold_padded"]
     B, H, S = c["B"], c["H"], c["S"]
     ms_ = 128 * wl.ceil_div(S, 128)
     SB = ms_ // 128
-    g = torch.Generator(device=dev)
-    g.manual_seed(seed)
-    mask = (torch.rand((B, H, SB, ms_), device=dev, generator=g) < c["keep"]).to(torch.int32)
+    if mask is None:
+        mask = _iid_mask(dev, seed)
     kvi = torch.full((B, H, SB, ms_), ms_, dtype=torch.int32, device=dev)
     kvn = torch.zeros((B, H, SB), dtype=torch.int32, device=dev)
 
@@ -146,20 +172,20 @@ def bench_compaction(dev, steps, warmup, seed=0):
 
     ms, _ = time_steps(step, steps, warmup)
     kept = int(kvn.sum().item())
+    assert torch.equal(kvn, (mask[..., :S] > 0).sum(-1).to(torch.int32)), "compaction counts differ from the mask's row sums"
     nbytes = 4.0 * B * H * SB * ms_ + 4.0 * kept + 4.0 * B * H * SB
     return dict(ms=ms, bytes=nbytes, kept=kept, shape=[B, H, SB, ms_])
 
 
-def bench_packed(dev, steps, warmup, seed=0):
+def bench_packed(dev, steps, warmup, seed=0, mask=None):
     """The bit-packed mask cache at the same mask: pack_mask (int32 votes -> bits) and
     packedmask_to_indexmask (bits -> index lists, the fused unpack + compaction)."""
     c = wl.CONFIGS["cfg4_threshold_padded"]
     B, H, S = c["B"], c["H"], c["S"]
     ms_ = 128 * wl.ceil_div(S, 128)
     SB = ms_ // 128
-    g = torch.Generator(device=dev)
-    g.manual_seed(seed)
-    mask = (torch.rand((B, H, SB, ms_), device=dev, generator=g) < c["keep"]).to(torch.int32)
+    if mask is None:
+        mask = _iid_mask(dev, seed)
     packed = torch.empty((B, H, SB, ms_ // 8), dtype=torch.uint8, device=dev)
     kvi = torch.full((B, H, SB, ms_), ms_, dtype=torch.int32, device=dev)
     kvn = torch.zeros((B, H, SB), dtype=torch.int32, device=dev)
@@ -227,6 +253,110 @@ def bench_sweeps(dev, steps, warmup, seed=0, heads=None):
     return dict(ms_maxq_denom=ms1, ms_booleanmask=ms2, flops=flops, mask_bytes=4.0 * mask.numel())
 
 
+def bench_cfg4_end_to_end(dev, steps, warmup, seed=0):
+    """The padded threshold path at B=1 H=24 N=32760 d=64 on ONE set of seeded clustered inputs, stage
+    by stage as the reference's caller runs it (python/spattn/sparseattn_functionals.py:95-114):
+    dense attention with row statistics -> threshold sweep -> lists -> sparse attention.  The
+    threshold is found on the device (untimed bisection) so that about 8 % of the (128-row q-block,
+    64-key block) pairs are kept.  Three routes from the statistics to the attention:
+      tokens    booleanmask_128 (int32 votes) -> booleanmask_to_indexmask -> sp_attn, 128-row q-blocks
+                (the reference's own sequence)
+      blocks128 bit-packed sweep -> block lists -> sp_attn_blocks, 128-row q-blocks
+      blocks64  the same with a mask row and a list per 64 query rows
+    Every attention launch uses the work order computed (untimed here, timed on its own) from its counts."""
+    c = wl.CONFIGS["cfg4_threshold_padded"]
+    B, H, S, D = c["B"], c["H"], c["S"], c["D"]
+    q, k, v = (t.to(dev) for t in wl.clustered_qkv(B, H, S, D, seed=seed))
+    Sp = 128 * wl.ceil_div(S, 128)
+    SB, nb = Sp // 128, Sp // 64
+    mx = torch.empty((B, H, 1, Sp), device=dev)
+    dn = torch.empty((B, H, 1, Sp), device=dev)
+    o = torch.empty_like(q)
+    out = {"workload": "cfg4: B=1 H=24 N=32760 (rows of 32768) d=64 bf16, K = N(0,1) + per-64-key-block offsets of sigma 1.5"}
+    n_sw = max(2, steps // 10)
+    ms, _ = time_steps(lambda: capi.fullattn_maxq_denom(o, mx, dn, q, k, v), n_sw, 1)
+    dense_flops = 4.0 * B * H * float(S) * S * D
+    out["fullattn_maxq_denom"] = {"ms": ms, "tflops": dense_flops / ms / 1e9, "mfma_frac": dense_flops / ms / 1e9 / PEAK_BF16_TFLOPS}
+    ms, _ = time_steps(lambda: capi.maxq_denom(mx, dn, q, k), n_sw, 1)
+    sweep_flops = 2.0 * B * H * float(Sp) * Sp * D
+    out["maxq_denom"] = {"ms": ms, "tflops": sweep_flops / ms / 1e9, "mfma_frac": sweep_flops / ms / 1e9 / PEAK_BF16_TFLOPS}
+
+    # threshold: bisection on log(tau) against the kept-block density of the 128-row block mask
+    pk = torch.empty((B, H, SB, Sp // 8), dtype=torch.uint8, device=dev)
+    bi = torch.full((B, H, SB, nb), -1, dtype=torch.int32, device=dev)
+    bc = torch.zeros((B, H, SB), dtype=torch.int32, device=dev)
+    nkb = wl.ceil_div(S, 64)
+
+    def density(tau):
+        capi.booleanmask_packed(pk, mx, dn, q, k, tau, qblk=128)
+        capi.packedmask_to_blocklists(bi, bc, pk, S)
+        return float(bc.float().mean().item()) / nkb
+
+    lo, hi = -40.0, 0.0
+    for _ in range(24):
+        mid = 0.5 * (lo + hi)
+        if density(float(np.exp(mid))) > c["keep"]:
+            lo = mid
+        else:
+            hi = mid
+    tau = float(np.exp(0.5 * (lo + hi)))
+    out["threshold"] = tau
+    out["block_density_q128"] = density(tau)
+
+    rows = B * H * SB
+    # route 1: the reference's sequence on int32 votes and key lists
+    mask = torch.zeros((B, H, SB, Sp), dtype=torch.int32, device=dev)
+    ms_sweep, _ = time_steps(lambda: capi.booleanmask_128(mask, mx, dn, q, k, tau), n_sw, 1)
+    cp = bench_compaction(dev, steps, warmup, mask=mask)
+    kvi = torch.full((B, H, SB, Sp), Sp, dtype=torch.int32, device=dev)
+    kvn = torch.zeros((B, H, SB), dtype=torch.int32, device=dev)
+    capi.booleanmask_to_indexmask(kvi, kvn, mask, S)
+    order = torch.empty((rows,), dtype=torch.int32, device=dev)
+    ms_order, _ = time_steps(lambda: capi.qblock_order(order, kvn), steps, warmup)
+    n_at = max(2, steps // 4)
+    ms_attn, _ = time_steps(lambda: capi.sp_attn(o, q, k, v, kvi, kvn, qblk=128, order=order), n_at, 2)
+    kept_keys = int(kvn.sum().item())
+    tok_flops = 4.0 * kept_keys * 128 * D
+    gb = cp["bytes"] / cp["ms"] / 1e6
+    out["tokens"] = {
+        "booleanmask_128_ms": ms_sweep, "booleanmask_128_tflops": sweep_flops / ms_sweep / 1e9,
+        "booleanmask_128_mfma_frac": sweep_flops / ms_sweep / 1e9 / PEAK_BF16_TFLOPS,
+        "booleanmask_128_write_gbps": 4.0 * mask.numel() / ms_sweep / 1e6,
+        "booleanmask_to_indexmask_ms": cp["ms"], "booleanmask_to_indexmask_gbps": gb,
+        "booleanmask_to_indexmask_hbm_frac": gb / PEAK_HBM_GBPS, "booleanmask_to_indexmask_bytes": cp["bytes"],
+        "qblock_order_ms": ms_order, "sp_attn_ms": ms_attn, "kept_keys": kept_keys,
+        "key_density": kept_keys / (float(rows) * S), "sp_attn_tflops": tok_flops / ms_attn / 1e9,
+        "sp_attn_mfma_frac": tok_flops / ms_attn / 1e9 / PEAK_BF16_TFLOPS,
+        "prepass_plus_attention_ms": ms_sweep + cp["ms"] + ms_order + ms_attn}
+    pkres = bench_packed(dev, steps, warmup, mask=mask)
+    out["mask_cache"] = pkres
+    del kvi, mask
+    # routes 2 and 3: bits and block lists
+    for qblk in (128, 64):
+        nq = wl.ceil_div(S, qblk)
+        pkq = torch.empty((B, H, nq, Sp // 8), dtype=torch.uint8, device=dev)
+        biq = torch.full((B, H, nq, nb), -1, dtype=torch.int32, device=dev)
+        bcq = torch.zeros((B, H, nq), dtype=torch.int32, device=dev)
+        ms_sw, _ = time_steps(lambda: capi.booleanmask_packed(pkq, mx, dn, q, k, tau, qblk=qblk), n_sw, 1)
+        ms_bl, _ = time_steps(lambda: capi.packedmask_to_blocklists(biq, bcq, pkq, S), steps, warmup)
+        kept = int(bcq.sum().item())
+        ordq = torch.empty((bcq.numel(),), dtype=torch.int32, device=dev)
+        capi.qblock_order(ordq, bcq)
+        ms_at, _ = time_steps(lambda: capi.sp_attn_blocks(o, q, k, v, biq, bcq, qblk=qblk, order=ordq), n_at, 2)
+        fl = wl.kept_block_flops(kept, qblk, 64, D)
+        bl_bytes = pkq.numel() + 4.0 * kept + 4.0 * bcq.numel()
+        out["blocks%d" % qblk] = {
+            "booleanmask_packed_ms": ms_sw, "booleanmask_packed_tflops": sweep_flops / ms_sw / 1e9,
+            "booleanmask_packed_mfma_frac": sweep_flops / ms_sw / 1e9 / PEAK_BF16_TFLOPS, "mask_bytes": float(pkq.numel()),
+            "packedmask_to_blocklists_ms": ms_bl, "packedmask_to_blocklists_gbps": bl_bytes / ms_bl / 1e6,
+            "packedmask_to_blocklists_bytes": bl_bytes, "kept_blocks": kept, "block_density": kept / (float(bcq.numel()) * nkb),
+            "sp_attn_blocks_ms": ms_at, "sp_attn_blocks_tflops": fl / ms_at / 1e9,
+            "sp_attn_blocks_mfma_frac": fl / ms_at / 1e9 / PEAK_BF16_TFLOPS,
+            "prepass_plus_attention_ms": ms_sw + ms_bl + ms_order + ms_at}
+    assert torch.isfinite(o.float()).all().item(), "non-finite attention output"
+    return out
+
+
 def cpu_baseline(res, budget_s=15.0):
     """Dense-masked PyTorch attention on the host cores over a bounded sample of the
     headline workload: 2048-row slabs of successive heads until the time budget is used."""
@@ -272,7 +402,7 @@ def main(argv=None) -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-extras", action="store_true", help="only the headline kernel")
-    ap.add_argument("--only", default="", help="run one leg only: sparse|tokens|compact|dense|sweeps|copy|packed|topk|zipf (no JSON contract)")
+    ap.add_argument("--only", default="", help="run one leg only: sparse|tokens|compact|dense|sweeps|copy|packed|topk|zipf|zipf64|cfg4 (no JSON contract)")
     args = ap.parse_args(argv)
     if args.gpus != 1:
         print("bench.py: this library is single-GPU; run with --gpus 1 (got %d)" % args.gpus, file=sys.stderr)
@@ -286,7 +416,8 @@ def main(argv=None) -> int:
 
     if args.only:
         fn = {"sparse": bench_sparse, "compact": bench_compaction, "dense": bench_dense, "sweeps": bench_sweeps,
-              "copy": bench_copy, "packed": bench_packed, "tokens": bench_tokens, "topk": bench_topk, "zipf": bench_zipf}[args.only]
+              "copy": bench_copy, "packed": bench_packed, "tokens": bench_tokens, "topk": bench_topk, "zipf": bench_zipf,
+              "zipf64": bench_zipf_sparse, "cfg4": bench_cfg4_end_to_end}[args.only]
         r = fn(dev, args.steps, args.warmup)
         r.pop("tensors", None)
         print(json.dumps(r))
@@ -304,7 +435,8 @@ def main(argv=None) -> int:
                                "26 of 256 key blocks per row incl. diagonal, bf16 O + fp32 lse",
                    "kept_blocks": res["kept_blocks"], "flops_per_step": res["flops"]},
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_SPARSE_BYTES, "traffic_unit": "bytes",
+                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": measured_traffic("attn_fwd_kernel<128,64,KV_BLOCKS>"),
+                     "traffic_unit": "bytes",
                      "kernel": "attn_fwd_kernel<128,64,KV_BLOCKS>"},
     }
     if not args.no_extras:
@@ -313,20 +445,31 @@ def main(argv=None) -> int:
                               "kernel": "attn_fwd_kernel<128,64,KV_TOKENS>", "ms": tk["ms"],
                               "tflops": tk["flops"] / (tk["ms"] * 1e-3) / 1e12,
                               "mfma_frac": tk["flops"] / (tk["ms"] * 1e-3) / 1e12 / PEAK_BF16_TFLOPS}
+        def zipf_entry(zp, what):
+            return {"workload": what, "mean_blocks": zp["mean_blocks"], "density": zp["density"],
+                    "saturated_rows": zp["saturated_rows"], "kept_blocks": zp["kept_blocks"],
+                    "ms_default_order": zp["ms_default"], "ms_longest_first": zp["ms_ordered"],
+                    "order_kernel_ms": zp["ms_order_kernel"],
+                    "tflops_longest_first": zp["flops"] / zp["ms_ordered"] / 1e9,
+                    "mfma_frac_longest_first": zp["flops"] / zp["ms_ordered"] / 1e9 / PEAK_BF16_TFLOPS}
+
         zp = bench_zipf(dev, max(2, args.steps // 4), 2)
-        out["zipf_lists"] = {"workload": "cfg5: B=1 H=8 N=65536 d=128, q-block 128, Zipf(1.2) block counts in [1,1024]",
-                             "ms_default_order": zp["ms_default"], "ms_longest_first": zp["ms_ordered"],
-                             "order_kernel_ms": zp["ms_order_kernel"],
-                             "tflops_longest_first": zp["flops"] / zp["ms_ordered"] / 1e9,
-                             "mfma_frac_longest_first": zp["flops"] / zp["ms_ordered"] / 1e9 / PEAK_BF16_TFLOPS}
-        cp = bench_compaction(dev, args.steps, args.warmup)
-        gbps = cp["bytes"] / (cp["ms"] * 1e-3) / 1e9
-        out["mask_pass"] = {"kernel": "compact_kernel (booleanmask_to_indexmask)", "workload": "cfg4 mask %s int32, %.1f%% kept"
-                            % (cp["shape"], 100.0 * cp["kept"] / np.prod(cp["shape"])), "ms": cp["ms"],
-                            "roofline": {"bound": "hbm", "achieved": gbps, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                                         "frac": gbps / PEAK_HBM_GBPS, "traffic": TRAFFIC_COMPACT_BYTES,
-                                         "traffic_unit": "bytes", "algorithmic_bytes": cp["bytes"]}}
-        pk = bench_packed(dev, args.steps, args.warmup)
+        out["zipf_lists"] = zipf_entry(zp, "cfg5 as its distribution is stated: B=1 H=8 N=65536 d=128, q-block 128, block counts "
+                                           "~ Zipf(1.2) clipped to [1,1024] (mean 28 % of the 1024 key blocks, a fifth of the rows at the clip)")
+        zs = bench_zipf_sparse(dev, max(2, args.steps // 4), 2)
+        out["zipf_lists_3pct"] = zipf_entry(zs, "cfg5 at its stated mean density: the same Zipf(1.2) counts clipped to [1,64] "
+                                                "(mean 3 % of the 1024 key blocks)")
+        e2e = bench_cfg4_end_to_end(dev, args.steps, args.warmup)
+        tk4 = e2e["tokens"]
+        out["mask_pass"] = {"kernel": "compact_kernel (booleanmask_to_indexmask)",
+                            "workload": "cfg4 vote mask [1, 24, 256, 32768] int32 of the threshold sweep (kept keys in runs), "
+                                        "%.1f%% of the keys kept" % (100.0 * tk4["key_density"]),
+                            "ms": tk4["booleanmask_to_indexmask_ms"],
+                            "roofline": {"bound": "hbm", "achieved": tk4["booleanmask_to_indexmask_gbps"], "peak": PEAK_HBM_GBPS,
+                                         "unit": "GB/s", "frac": tk4["booleanmask_to_indexmask_hbm_frac"],
+                                         "traffic": measured_traffic("compact_kernel"), "traffic_unit": "bytes",
+                                         "algorithmic_bytes": tk4["booleanmask_to_indexmask_bytes"]}}
+        pk = e2e.pop("mask_cache")
         out["mask_cache"] = {
             "workload": "same mask, bit-packed (1 bit per key)",
             "pack_mask_ms": pk["ms_pack"], "pack_mask_gbps": pk["bytes_pack"] / pk["ms_pack"] / 1e6,
@@ -334,6 +477,7 @@ def main(argv=None) -> int:
             "packedmask_to_indexmask_ms": pk["ms_index"], "packedmask_to_indexmask_gbps": pk["bytes_index"] / pk["ms_index"] / 1e6,
             "packedmask_to_indexmask_hbm_frac": pk["bytes_index"] / pk["ms_index"] / 1e6 / PEAK_HBM_GBPS,
             "algorithmic_bytes": [pk["bytes_pack"], pk["bytes_index"]]}
+        out["cfg4_end_to_end"] = e2e
         tp = bench_topk(dev, max(2, args.steps // 4), 2)
         out["topk_mask"] = {"workload": "cfg4 shape, q-block-mean top-k, %d keys per q-block" % tp["select_k"],
                             "ms": tp["ms"], "gbps": tp["bytes"] / tp["ms"] / 1e6,
@@ -342,12 +486,6 @@ def main(argv=None) -> int:
         out["dense_full_attn"] = {"workload": "cfg2: B=4 H=16 N=4096 d=64", "ms": dn["ms"],
                                   "tflops": dn["flops"] / (dn["ms"] * 1e-3) / 1e12,
                                   "mfma_frac": dn["flops"] / (dn["ms"] * 1e-3) / 1e12 / PEAK_BF16_TFLOPS}
-        sw = bench_sweeps(dev, max(2, args.steps // 10), 1)
-        out["prepass_sweeps"] = {
-            "workload": "cfg4: B=1 H=24 N=32760 d=64",
-            "maxq_denom_ms": sw["ms_maxq_denom"], "maxq_denom_tflops": sw["flops"] / sw["ms_maxq_denom"] / 1e9,
-            "booleanmask_128_ms": sw["ms_booleanmask"], "booleanmask_128_tflops": sw["flops"] / sw["ms_booleanmask"] / 1e9,
-            "booleanmask_128_write_gbps": sw["mask_bytes"] / sw["ms_booleanmask"] / 1e6}
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(res)
     else:
