@@ -32,6 +32,8 @@ _SIGNATURES = {
     "spattn_sp_attn_blocks": (_c_int, [_c_void_p] * 7 + [_c_int] * 7 + [_c_float, _c_void_p]),
     "spattn_sp_attn_ordered": (_c_int, [_c_void_p] * 8 + [_c_int] * 7 + [_c_float, _c_void_p]),
     "spattn_sp_attn_blocks_ordered": (_c_int, [_c_void_p] * 8 + [_c_int] * 7 + [_c_float, _c_void_p]),
+    "spattn_sp_attn_blocks_balanced": (_c_int, [_c_void_p] * 7 + [_c_int] * 7 + [_c_float, _c_void_p]),
+    "spattn_init": (_c_int, []),
     "spattn_qblock_order": (_c_int, [_c_void_p] * 2 + [_c_int, _c_void_p]),
     "spattn_all_index_mask": (_c_int, [_c_void_p] * 2 + [_c_int] * 5 + [_c_void_p]),
     "spattn_fullattn_maxq_denom": (_c_int, [_c_void_p] * 6 + [_c_int] * 5 + [_c_float, _c_void_p]),
@@ -163,6 +165,24 @@ def sp_attn_blocks(o, q, k, v, blk_indices, blk_counts, *, lse=None, qblk=None, 
                                                 _ptr(v, bf16), _ptr(blk_indices, i32), _ptr(blk_counts, i32),
                                                 _ptr(order, i32), int(blk_indices.shape[3]), qblk, B, H, S, D, kv_len,
                                                 scale, _stream(stream)))
+
+
+BALANCED_MAX_QBLOCKS = 1 << 20
+
+
+def sp_attn_blocks_balanced(o, q, k, v, blk_indices, blk_counts, *, lse=None, qblk=None, kv_len=0, scale=0.0, stream=None):
+    """sp_attn_blocks in longest-list-first order with the order kept in the library's own device
+    array: allocates nothing.  Calls that overlap on one device race on that array."""
+    B, H, S, D = _bhsd(q)
+    if blk_indices.dim() != 4:
+        raise ValueError("blk_indices must be [B,H,SB,max_blocks]")
+    if qblk is None:
+        qblk = infer_qblk(S, int(blk_indices.shape[2]))
+    if blk_counts.numel() != B * H * int(blk_indices.shape[2]):
+        raise ValueError("blk_counts must have B*H*SB entries")
+    _check(load().spattn_sp_attn_blocks_balanced(_ptr(o, bf16), _ptr(lse, f32), _ptr(q, bf16), _ptr(k, bf16), _ptr(v, bf16),
+                                                 _ptr(blk_indices, i32), _ptr(blk_counts, i32), int(blk_indices.shape[3]),
+                                                 qblk, B, H, S, D, kv_len, scale, _stream(stream)))
 
 
 def qblock_order(order, counts, *, stream=None):

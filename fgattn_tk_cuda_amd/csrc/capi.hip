@@ -3,6 +3,8 @@
 
 #include <math.h>
 
+#include <mutex>
+
 #include "dispatch.h"
 
 namespace {
@@ -258,6 +260,73 @@ int spattn_sp_attn_blocks_ordered(void* o, float* lse, const void* q, const void
   return from_hip(spattn::run_attn_blocks(p, D, qblk, as_stream(stream)));
 }
 
+// ---- block-list attention in balanced order without a caller-provided order buffer -------------
+// The work order (one int per q-block) lives in a device array that belongs to the library:
+// every device the library runs on holds its own copy of it, at its own address, until the
+// process ends.  Host code never uses the array's name as an address: the per-device address is
+// looked up once with hipGetSymbolAddress and kept.
+
+}  // extern "C"
+
+namespace {
+
+constexpr int kScratchInts = SPATTN_BALANCED_MAX_QBLOCKS;
+static __device__ __align__(256) int scratch[kScratchInts];
+
+std::mutex g_scratch_mu;
+int* g_scratch_ptr[spattn::kMaxDevices] = {};
+
+// Address of `scratch` on the current device (looked up on the first call per device).
+int scratch_on_current_device(int** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= spattn::kMaxDevices) return SPATTN_ERR_SHAPE;
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (p == nullptr) return (int)hipErrorInvalidSymbol;
+    g_scratch_ptr[dev] = static_cast<int*>(p);
+  }
+  *out = g_scratch_ptr[dev];
+  return SPATTN_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int spattn_init(void) {
+  int* p = nullptr;
+  return done(scratch_on_current_device(&p));
+}
+
+int spattn_sp_attn_blocks_balanced(void* o, float* lse, const void* q, const void* k, const void* v,
+                                   const int* blk_indices, const int* blk_counts, int max_blocks, int qblk, int B, int H,
+                                   int S, int D, int kv_len, float scale, void* stream) {
+  if (int st = check_qkv(q, k, B, H, S, D)) return done(st);
+  if (!o || !v || !blk_indices || !blk_counts) return done(SPATTN_ERR_NULL);
+  if (misaligned(o) || misaligned(v)) return done(SPATTN_ERR_ALIGN);
+  if (qblk != 64 && qblk != 128) return done(SPATTN_ERR_QBLK);
+  if (max_blocks <= 0) return done(SPATTN_ERR_SHAPE);
+  const long long nq = (long long)B * H * ((S + qblk - 1) / qblk);
+  if (nq > kScratchInts) return done(SPATTN_ERR_SCRATCH);
+  int* order = nullptr;
+  if (int st = scratch_on_current_device(&order)) return done(st);
+  // the order kernel writes all nq entries it is asked for: nothing of an earlier call is read
+  const hipError_t e = spattn::run_qblock_order(order, blk_counts, (int)nq, as_stream(stream));
+  if (e != hipSuccess) return from_hip(e);
+  spattn::AttnParams p = base_params(q, k, v, o, B, H, S, D, kv_len, scale, qblk);
+  p.lse = lse;
+  p.idx = blk_indices;
+  p.cnt = blk_counts;
+  p.idx_stride = max_blocks;
+  p.order = order;
+  return from_hip(spattn::run_attn_blocks(p, D, qblk, as_stream(stream)));
+}
+
 // ---- the reference's binding surface: default stream, default scale, q-block 128 ----
 
 void attn_fwd_wg_impl(void* o, void* q, void* k, void* v, int batch, int heads, int seq, int D) {
@@ -306,6 +375,7 @@ const char* spattn_status_string(int status) {
     case SPATTN_ERR_QBLK: return "q-block must be 64 or 128";
     case SPATTN_ERR_ALIGN: return "pointer is not 16-byte aligned";
     case SPATTN_ERR_SHAPE: return "a size is not positive or is inconsistent";
+    case SPATTN_ERR_SCRATCH: return "more q-blocks than the library's own work-order array holds";
     default: return status > 0 ? hipGetErrorString((hipError_t)status) : "unknown status";
   }
 }

@@ -29,6 +29,10 @@ extern "C" {
 #define SPATTN_ERR_QBLK -4       /* q-block is not 64 or 128 */
 #define SPATTN_ERR_ALIGN -5      /* a pointer is not 16-byte aligned */
 #define SPATTN_ERR_SHAPE -6      /* a size is not positive / inconsistent, or seq >= 2^24 */
+#define SPATTN_ERR_SCRATCH -7    /* more q-blocks than SPATTN_BALANCED_MAX_QBLOCKS */
+
+/* q-blocks (batch * heads * ceil(seq / qblk)) that spattn_sp_attn_blocks_balanced can order */
+#define SPATTN_BALANCED_MAX_QBLOCKS (1 << 20)
 
 /* ---- group 1: the reference's binding surface ------------------------------------ */
 
@@ -181,6 +185,22 @@ int spattn_sp_attn_ordered(void* o, float* lse, const void* q, const void* k, co
 int spattn_sp_attn_blocks_ordered(void* o, float* lse, const void* q, const void* k, const void* v,
                                   const int* blk_indices, const int* blk_counts, const int* order, int max_blocks,
                                   int qblk, int batch, int heads, int seq, int D, int kv_len, float scale, void* stream);
+
+/* Block-list attention in balanced (longest list first) order for callers that cannot
+ * allocate: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * It has no counterpart in the reference.  It is spattn_qblock_order followed by
+ * spattn_sp_attn_blocks_ordered, bit for bit, with the work order kept in a device array that
+ * belongs to the library (4 MiB per device, held until the process ends) instead of a buffer
+ * the caller provides; it calls no allocating routine.  At most SPATTN_BALANCED_MAX_QBLOCKS
+ * q-blocks, else SPATTN_ERR_SCRATCH and nothing is launched.  All calls on one device share
+ * that array: calls that overlap on one device (two streams, two threads) race on it - run
+ * them one after the other, or use the _ordered form with a buffer per stream.
+ * spattn_init looks the array's address up for the current device; optional, the first call
+ * on a device does the same (call it before a graph capture starts). */
+int spattn_init(void);
+int spattn_sp_attn_blocks_balanced(void* o, float* lse, const void* q, const void* k, const void* v,
+                                   const int* blk_indices, const int* blk_counts, int max_blocks, int qblk, int batch,
+                                   int heads, int seq, int D, int kv_len, float scale, void* stream);
 
 /* Status of the most recent call on this host thread, and its text. */
 int spattn_last_status(void);
