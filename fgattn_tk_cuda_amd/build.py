@@ -74,6 +74,17 @@ def build_lib(verbose: bool = True) -> Path:
     return LIB
 
 
+PROBES = PKG / "libspattn_probes.so"
+
+
+def build_probes(verbose: bool = True) -> Path:
+    """Compile the roofline probes (csrc/probes.hip) into libspattn_probes.so; bench.py --only ldsprobe runs them."""
+    _run([_hipcc(), *HIPCC_FLAGS, "-shared", "-o", str(PROBES), str(CSRC / "probes.hip")])
+    if verbose:
+        print("built", PROBES)
+    return PROBES
+
+
 def ext_path() -> Path:
     import sysconfig
 
@@ -115,6 +126,7 @@ def main(argv=None) -> int:
     build_lib()
     if not args.lib_only:
         build_torch_ext()
+        build_probes()
     return 0
 
 
