@@ -94,7 +94,7 @@ typedef SPATTN_LDS const unsigned char* lds_cptr;
 // bookkeeping (with the builtin it drains every outstanding load before each LDS read),
 // so the waits are placed by hand.
 __device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(gptr) : "memory");
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(gptr) : "memory", "m0");
 }
 // Same with a wave-uniform base pointer and a 32-bit per-lane byte offset.
 // The base goes through readfirstlane: under scalar-register pressure the compiler may keep
@@ -104,7 +104,7 @@ __device__ __forceinline__ void dma16(const void* sbase, uint32_t voff, uint32_t
   const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)b);
   const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
   const uint64_t sb = ((uint64_t)hi << 32) | lo;
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(voff), "s"(sb) : "memory");
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(voff), "s"(sb) : "memory", "m0");
 }
 // 16-byte global load that the compiler does not count either: the destination is valid only
 // behind a hand-placed vmcnt wait, after which the caller ties the registers to that point with
