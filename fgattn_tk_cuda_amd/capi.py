@@ -43,6 +43,9 @@ _SIGNATURES = {
     "spattn_booleanmask_packed": (_c_int, [_c_void_p, _c_float, _c_int, _c_int] + [_c_void_p] * 4 + [_c_int] * 5 + [_c_float, _c_void_p]),
     "spattn_packedmask_to_blocklists": (_c_int, [_c_void_p] * 4 + [_c_int] * 6 + [_c_void_p]),
     "spattn_booleanmask_to_blocklists": (_c_int, [_c_void_p] * 4 + [_c_int] * 6 + [_c_void_p]),
+    "spattn_maxq_denom_blockmax": (_c_int, [_c_void_p] * 5 + [_c_int] * 5 + [_c_float, _c_void_p]),
+    "spattn_fullattn_maxq_denom_blockmax": (_c_int, [_c_void_p] * 7 + [_c_int] * 5 + [_c_float, _c_void_p]),
+    "spattn_blockmax_to_blocklists": (_c_int, [_c_void_p] * 6 + [_c_float] + [_c_int] * 6 + [_c_float, _c_int, _c_void_p]),
     "spattn_pack_mask": (_c_int, [_c_void_p] * 2 + [_c_int] * 4 + [_c_void_p]),
     "spattn_packedmask_to_indexmask": (_c_int, [_c_void_p] * 3 + [_c_int] * 5 + [_c_void_p]),
     "spattn_qk_topkmask_indices": (_c_int, [_c_void_p] * 6 + [_c_int] * 9 + [_c_void_p]),
@@ -274,6 +277,51 @@ def booleanmask_to_blocklists(blk_indices, blk_counts, booleanmask, seq, *, bloc
     _check(load().spattn_booleanmask_to_blocklists(_ptr(blk_indices, i32), _ptr(blk_counts, i32),
                                                    _ptr(blockmask, torch.uint8), _ptr(booleanmask, i32), B, H, int(seq),
                                                    SB, MS, int(blk_indices.shape[3]), _stream(stream)))
+
+
+def _need_blockmax(blockmax, B, H, S):
+    sp = 128 * ((S + 127) // 128)
+    if blockmax.numel() != B * H * (sp // 64) * sp:
+        raise ValueError("blockmax must be fp32 [B,H,%d,%d]" % (sp // 64, sp))
+
+
+def maxq_denom_blockmax(max_q, denom, blockmax, q, k, *, kv_len=0, scale=0.0, stream=None):
+    """maxq_denom that also writes blockmax fp32 [B,H,Sp/64,Sp]: [J][r] = max of q[r].k[c] over the keys c < kv_len
+    of 64-key block J (blocks without such a key are left as they are)."""
+    B, H, S, D = _bhsd(q)
+    _need_padded(max_q, denom, B, H, S)
+    _need_blockmax(blockmax, B, H, S)
+    _check(load().spattn_maxq_denom_blockmax(_ptr(max_q, f32), _ptr(denom, f32), _ptr(blockmax, f32), _ptr(q, bf16),
+                                             _ptr(k, bf16), B, H, S, D, kv_len, scale, _stream(stream)))
+
+
+def fullattn_maxq_denom_blockmax(o, max_q, denom, blockmax, q, k, v, *, kv_len=0, scale=0.0, stream=None):
+    """fullattn_maxq_denom with the blockmax output of maxq_denom_blockmax."""
+    B, H, S, D = _bhsd(q)
+    _need_padded(max_q, denom, B, H, S)
+    _need_blockmax(blockmax, B, H, S)
+    _check(load().spattn_fullattn_maxq_denom_blockmax(_ptr(o, bf16), _ptr(max_q, f32), _ptr(denom, f32),
+                                                      _ptr(blockmax, f32), _ptr(q, bf16), _ptr(k, bf16), _ptr(v, bf16),
+                                                      B, H, S, D, kv_len, scale, _stream(stream)))
+
+
+def blockmax_to_blocklists(blk_indices, blk_counts, blockmax, max_q, denom, threshold, seq, D, *, qblk=128,
+                           blockmask=None, kv_len=0, scale=0.0, stream=None):
+    """Threshold test on the block maxima of a statistics sweep -> ascending 64-key block lists per
+    q-block of qblk rows (and, optionally, the block mask uint8 [B,H,ceil(S/qblk),Sp/64])."""
+    if blk_indices.dim() != 4:
+        raise ValueError("blk_indices must be [B,H,ceil(S/qblk),max_blocks]")
+    B, H, SB, MB = (int(x) for x in blk_indices.shape)
+    S = int(seq)
+    if qblk not in (64, 128) or SB != (S + qblk - 1) // qblk:
+        raise ValueError("blk_indices must hold ceil(S/qblk) lists per head, qblk 64 or 128")
+    _need_padded(max_q, denom, B, H, S)
+    _need_blockmax(blockmax, B, H, S)
+    _blocklist_args(blk_indices, blk_counts, blockmask, B, H, SB, 128 * ((S + 127) // 128))
+    _check(load().spattn_blockmax_to_blocklists(_ptr(blk_indices, i32), _ptr(blk_counts, i32),
+                                                _ptr(blockmask, torch.uint8), _ptr(blockmax, f32), _ptr(max_q, f32),
+                                                _ptr(denom, f32), float(threshold), int(qblk), B, H, S, int(D), kv_len,
+                                                scale, MB, _stream(stream)))
 
 
 def pack_mask(packed, booleanmask, *, stream=None):

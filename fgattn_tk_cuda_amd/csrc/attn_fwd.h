@@ -424,16 +424,23 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     mloc = fmaxf(mloc, fmaxf(s[mb][r], s[mb][r + 1]));
     mloc = fmaxf(mloc, fmaxf(s[mb][r + 2], s[mb][r + 3]));
   };
-  auto stat_finish = [&](float mloc) -> float {
+  // tile: the key block the maxima belong to.  With the statistics outputs a caller may also ask
+  // for them per key block (blockmax[J][row], raw like max_q): the threshold test of the mask
+  // pre-pass, softmax(r, c) > tau, holds for some key of block J exactly when the block's maximum
+  // passes it, so these S x S/64 numbers replace the second score sweep for block-level masks.
+  auto stat_finish = [&](float mloc, int tile) -> float {
     mloc = pair_max(mloc);
+    if constexpr (STATS && KSPLIT == 1 && MODE == KV_DENSE) {
+      if (p.blockmax != nullptr && g == 0) p.blockmax[((size_t)bh * (p.Sp >> 6) + tile) * p.Sp + qrow] = mloc;
+    }
     m_true = fmaxf(m_true, mloc);
     return mloc * p.sf;
   };
-  auto row_stats = [&](const f32x16 (&s)[NMB]) -> float {
+  auto row_stats = [&](const f32x16 (&s)[NMB], int tile) -> float {
     float mloc;
 #pragma unroll
     for (int k = 0; k < NP; ++k) stat_piece(s, k, mloc);
-    return stat_finish(mloc);
+    return stat_finish(mloc, tile);
   };
   // Move the exponent reference if some row of the wave outgrew it; rescales O and l.
   auto maybe_rescale = [&](float mloc_sf) {
@@ -490,7 +497,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   auto softmax_close = [&](const f32x16 (&s)[NMB], int par) {
     if constexpr (LAZY_MAX) {
       if (__any(!(l_tile <= kTrigger))) {
-        maybe_rescale(row_stats(s));
+        maybe_rescale(row_stats(s, 0));
         // a row that still has no reference has seen masked keys only: p = exp2(-inf - 0) = 0
         softmax_only(s, par, mr_sf == kNegInf ? 0.f : mr_sf);
       }
@@ -599,7 +606,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   // EARLY_SM: the exponentials of registers 0-7 of s_next (the tile after, parity par ^ 1) are
   // taken between the multiplies.
   auto pv_tile = [&](auto first_loaded, auto stat_c, uint32_t vofs, const TileLoad* tl, bool live, const f32x16 (&s_next)[NMB],
-                     int par, auto early_sm) -> float {
+                     int par, auto early_sm, int tile_next = 0) -> float {
     constexpr bool STAT = decltype(stat_c)::value;
     constexpr bool EARLY_SM = decltype(early_sm)::value;
     constexpr int MPP = NDB / 2;   // EARLY_SM: multiplies per pair of score registers
@@ -646,7 +653,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
 #pragma unroll
       for (int k = 0; k < NP; ++k) stat_piece(s_next, k, mloc);
     }
-    if constexpr (STAT) return stat_finish(mloc);
+    if constexpr (STAT) return stat_finish(mloc, tile_next);
     return 0.f;
   };
 
@@ -697,9 +704,9 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     if constexpr (HAS_V) {
       const TileLoad tl_second = K_FIRST ? prepare_tile(d_v, VN, true, GV{}) : prepare_tile(d_k, KN, false, GK{});
       mloc_sf = pv_tile(std::true_type{}, stat_t{}, VS * TILE, &tl_second, K_FIRST ? true : has_kn, s_b, PAR,
-                        std::integral_constant<bool, SPLIT_SM>{});
+                        std::integral_constant<bool, SPLIT_SM>{}, it + 1);
     } else {
-      mloc_sf = pv_tile(std::true_type{}, stat_t{}, 0, nullptr, false, s_b, PAR, std::false_type{});
+      mloc_sf = pv_tile(std::true_type{}, stat_t{}, 0, nullptr, false, s_b, PAR, std::false_type{}, it + 1);
     }
     if constexpr (!LAZY_MAX) maybe_rescale(mloc_sf);
   };
@@ -726,7 +733,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     qk_tile(std::false_type{}, std::false_type{}, 0, 0, s_e, s_e, 0, nullptr, false);
     if constexpr (MODE == KV_TOKENS) mask_tile(idw[0], idh[0], s_e);
     else mask_tile(hd[0], 0, s_e);
-    maybe_rescale(row_stats(s_e));
+    maybe_rescale(row_stats(s_e, 0));
     if constexpr (SPLIT_SM) softmax_half(s_e, 0, 0);   // nothing to hide these under
 
     int it = 0;

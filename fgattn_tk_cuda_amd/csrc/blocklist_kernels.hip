@@ -11,6 +11,8 @@
 // reference's int32 vote mask (a pure HBM stream like the per-key compaction).  One wave owns
 // one row; a lane stands for one block of a group of 64, so the rank of a kept block is a
 // wave ballot and a bit count - no atomics, deterministic, ascending.
+#include <math.h>
+
 #include "common.h"
 #include "dispatch.h"
 
@@ -102,6 +104,81 @@ __global__ __launch_bounds__(256) void votes_to_blocklists_kernel(int* __restric
   }
 }
 
+// Block maxima -> block lists: the threshold test of the mask pre-pass on the per-(row, key block)
+// score maxima that the statistics sweep writes next to max_q and denom (blockmax[b][h][J][r],
+// raw scores).  Some key c of block J passes  exp2((s[r,c] - max_q[r]) sf) / denom[r] > thresh
+// (include/mask_utils.cuh:231-238) exactly when the block's maximum does, so
+//   MB[I, J] = OR_{r in q-block I, r < seq} ( blockmax[J][r] > t[r] ),
+//   t[r] = (log2 thresh + max_q[r] sf + log2 denom[r]) / sf   (the sweep kernel's per-row constant),
+// is the block mask of the threshold sweep without a second pass over Q K^T: one read of
+// 4 Sp Sp/64 bytes per head instead of 2 Sp^2 D flops.  One wave owns one q-block (QB rows, a lane
+// holds one or two of them); per key block a 256- or 512-byte line of maxima is compared and the
+// votes of the wave are one ballot; kept blocks are appended 64 at a time as in the kernels above.
+template <int QB>
+__global__ __launch_bounds__(256) void blockmax_to_blocklists_kernel(int* __restrict__ blk_indices,
+                                                                    int* __restrict__ blk_counts,
+                                                                    unsigned char* __restrict__ blockmask,
+                                                                    const float* __restrict__ blockmax,
+                                                                    const float* __restrict__ max_q,
+                                                                    const float* __restrict__ denom, float log2_thresh,
+                                                                    float sf, int heads_total, int S, int Sp, int kv_len,
+                                                                    int max_blocks, int bm_stride) {
+  constexpr int RPL = QB / 64;   // rows per lane
+  constexpr int U = 16;          // key blocks in flight per wave
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int nqb = (S + QB - 1) / QB;
+  const int rows = heads_total * nqb;
+  const int nblk = (kv_len + 63) >> 6;    // key blocks that hold a key
+  const int nbs = Sp >> 6;                // block rows of a head in blockmax
+  const float inv_sf = 1.f / sf;
+  for (int row = blockIdx.x * 4 + wave; row < rows; row += gridDim.x * 4) {
+    const int bh = row / nqb, I = row - bh * nqb;
+    float t[RPL];
+    int r[RPL];
+#pragma unroll
+    for (int j = 0; j < RPL; ++j) {
+      r[j] = I * QB + 64 * j + lane;
+      t[j] = __builtin_huge_valf();   // a row that does not exist, or has no key, never votes
+      if (r[j] < S) {
+        const float mq = max_q[(size_t)bh * Sp + r[j]];
+        const float dn = denom[(size_t)bh * Sp + r[j]];
+        if (dn > 0.f) t[j] = (log2_thresh + (mq * sf + __log2f(dn))) * inv_sf;
+      }
+      r[j] = r[j] < Sp ? r[j] : Sp - 1;
+    }
+    const float* __restrict__ src = blockmax + (size_t)bh * nbs * Sp;
+    int* __restrict__ dst = blk_indices + (size_t)row * max_blocks;
+    unsigned char* mrow = blockmask ? blockmask + (size_t)row * bm_stride : nullptr;
+    int count = 0;
+    for (int J0 = 0; J0 < nblk; J0 += 64) {
+      unsigned long long word = 0;   // bit j: block J0 + j is kept
+#pragma unroll 1
+      for (int u0 = 0; u0 < 64 && J0 + u0 < nblk; u0 += U) {
+        float x[U][RPL];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int J = J0 + u0 + u;
+          const int Jc = J < nblk ? J : nblk - 1;
+#pragma unroll
+          for (int j = 0; j < RPL; ++j) x[u][j] = __builtin_nontemporal_load(src + (size_t)Jc * Sp + r[j]);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          bool f = x[u][0] > t[0];
+          if constexpr (RPL == 2) f = f || (x[u][1] > t[1]);
+          if (__ballot(f) != 0ull && J0 + u0 + u < nblk) word |= 1ull << (u0 + u);
+        }
+      }
+      append_blocks((word >> lane) & 1ull, J0 + lane, bm_stride, count, dst, mrow, max_blocks);
+    }
+    // block-mask entries behind the last key block of the head
+    if (mrow != nullptr)
+      for (int J = ((nblk + 63) & ~63) + lane; J < bm_stride; J += 64) mrow[J] = 0;
+    if (lane == 0) blk_counts[row] = count;
+  }
+}
+
 static int blocklist_grid(int rows) {
   int grid = (rows + 3) / 4;
   return grid > kBlockListMaxGrid ? kBlockListMaxGrid : grid;
@@ -120,6 +197,24 @@ hipError_t run_votes_to_blocklists(int* blk_indices, int* blk_counts, unsigned c
   if (rows <= 0) return hipSuccess;
   hipLaunchKernelGGL(votes_to_blocklists_kernel, dim3(blocklist_grid(rows)), dim3(256), 0, stream, blk_indices,
                      blk_counts, blockmask, votes, rows, mask_stride, kv_len, max_blocks);
+  return hipGetLastError();
+}
+
+hipError_t run_blockmax_to_blocklists(int* blk_indices, int* blk_counts, unsigned char* blockmask, const float* blockmax,
+                                      const float* max_q, const float* denom, float thresh, float sf, int qblk,
+                                      int heads_total, int S, int kv_len, int max_blocks, hipStream_t stream) {
+  const int nqb = (S + qblk - 1) / qblk;
+  const int rows = heads_total * nqb;
+  if (rows <= 0) return hipSuccess;
+  const int Sp = ((S + 127) / 128) * 128;
+  const float lt = thresh > 0.f ? log2f(thresh) : -__builtin_huge_valf();
+  const int grid = blocklist_grid(rows);
+  if (qblk == 128)
+    hipLaunchKernelGGL(blockmax_to_blocklists_kernel<128>, dim3(grid), dim3(256), 0, stream, blk_indices, blk_counts, blockmask,
+                       blockmax, max_q, denom, lt, sf, heads_total, S, Sp, kv_len, max_blocks, Sp >> 6);
+  else
+    hipLaunchKernelGGL(blockmax_to_blocklists_kernel<64>, dim3(grid), dim3(256), 0, stream, blk_indices, blk_counts, blockmask,
+                       blockmax, max_q, denom, lt, sf, heads_total, S, Sp, kv_len, max_blocks, Sp >> 6);
   return hipGetLastError();
 }
 

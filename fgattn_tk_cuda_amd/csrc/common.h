@@ -32,6 +32,7 @@ struct AttnParams {
   float* lse;         // optional fp32 [B,H,S], natural log
   float* max_q;       // optional fp32 [B,H,1,Sp], raw (unscaled) row max
   float* denom;       // optional fp32 [B,H,1,Sp]
+  float* blockmax;    // optional fp32 [B,H,Sp/64,Sp]: raw max of row r over the keys of block J at [J][r] (dense + statistics only)
   const int* idx;     // [B,H,SBq,idx_stride] token ids or block ids
   const int* cnt;     // [B*H*SBq]
   int idx_stride;
@@ -92,9 +93,11 @@ typedef SPATTN_LDS const unsigned char* lds_cptr;
 // One wave-wide HBM -> LDS copy: lane l's 16 bytes land at lds_base + 16 l.
 // Written as asm on purpose: the compiler does not count this load in its own vmcnt
 // bookkeeping (with the builtin it drains every outstanding load before each LDS read),
-// so the waits are placed by hand.
+// so the waits are placed by hand.  m0 cannot be named as clobbered (the compiler reserves it and
+// warns that such a clobber is not honoured); tests/test_asm_inflight_loads.py checks on the
+// listing that no compiler-generated instruction reads m0 across these statements.
 __device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(gptr) : "memory", "m0");
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(gptr) : "memory");
 }
 // Same with a wave-uniform base pointer and a 32-bit per-lane byte offset.
 // The base goes through readfirstlane: under scalar-register pressure the compiler may keep
@@ -104,7 +107,7 @@ __device__ __forceinline__ void dma16(const void* sbase, uint32_t voff, uint32_t
   const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)b);
   const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
   const uint64_t sb = ((uint64_t)hi << 32) | lo;
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(voff), "s"(sb) : "memory", "m0");
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(voff), "s"(sb) : "memory");
 }
 // 16-byte global load that the compiler does not count either: the destination is valid only
 // behind a hand-placed vmcnt wait, after which the caller ties the registers to that point with

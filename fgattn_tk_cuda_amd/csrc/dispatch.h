@@ -28,6 +28,10 @@ hipError_t run_packed_to_blocklists(int* blk_indices, int* blk_counts, unsigned 
 hipError_t run_votes_to_blocklists(int* blk_indices, int* blk_counts, unsigned char* blockmask, const int* votes,
                                    int rows, int mask_stride, int kv_len, int max_blocks, hipStream_t stream);
 
+hipError_t run_blockmax_to_blocklists(int* blk_indices, int* blk_counts, unsigned char* blockmask, const float* blockmax,
+                                      const float* max_q, const float* denom, float thresh, float sf, int qblk,
+                                      int heads_total, int S, int kv_len, int max_blocks, hipStream_t stream);
+
 // topk_kernels.hip
 hipError_t run_topk_mask(int* kv_indices, int* kv_num, uint16_t* score, uint16_t* qmean, const uint16_t* q,
                          const uint16_t* k, int B, int H, int S, int D, int blk, int kv_len, int select_k,

@@ -155,6 +155,32 @@ int spattn_booleanmask_to_blocklists(int* blk_indices, int* blk_counts, void* bl
                                      int batch, int heads, int seq, int seqblocks, int mask_stride, int max_blocks,
                                      void* stream);
 
+/* Block-level pre-pass without a second score sweep.  The statistics sweeps can also write, next
+ * to max_q and denom, the raw score maximum of every row over every 64-key block:
+ * blockmax fp32 [batch,heads,Sp/64,Sp] with Sp = 128*ceil(seq/128), entry [J][r] = max over the
+ * keys c of block J with c < kv_len of q[r].k[c] (blocks without such a key are not written).
+ * The reference's threshold test  exp2((s[r,c] - max_q[r]) sf) / denom[r] > threshold
+ * (include/mask_utils.cuh:231-238) holds for some key of block J exactly when it holds for the
+ * block's maximum, so spattn_blockmax_to_blocklists derives the block mask
+ *   MB[I,J] = OR_{r in q-block I, r < seq} ( blockmax[J][r] passes the test of row r )
+ * and the ascending block lists from 4*Sp*Sp/64 bytes per head instead of the 2*Sp*Sp*D flops of
+ * the sweep (include/mask_utils.cuh:131-243 + 273-302 for block-level masks); thresholds can be
+ * changed without another sweep.  qblk = 64 or 128 rows per list; outputs as
+ * spattn_packedmask_to_blocklists: blk_indices [batch,heads,ceil(seq/qblk),max_blocks] (entries
+ * behind the count keep the caller's fill), blk_counts [batch,heads,ceil(seq/qblk)], optional
+ * blockmask uint8 [batch,heads,ceil(seq/qblk),Sp/64].  max_q / denom are those of the same sweep
+ * ([batch,heads,1,Sp]); scale and kv_len must be the ones the sweep was given.
+ * The _blockmax sweeps replace maxq_denom_impl / attn_maxq_denom_impl
+ * (python/extension.cpp:22-33) with the extra output. */
+int spattn_maxq_denom_blockmax(float* max_q, float* denom, float* blockmax, const void* q, const void* k, int batch,
+                               int heads, int seq, int D, int kv_len, float scale, void* stream);
+int spattn_fullattn_maxq_denom_blockmax(void* o, float* max_q, float* denom, float* blockmax, const void* q, const void* k,
+                                        const void* v, int batch, int heads, int seq, int D, int kv_len, float scale,
+                                        void* stream);
+int spattn_blockmax_to_blocklists(int* blk_indices, int* blk_counts, void* blockmask, const float* blockmax,
+                                  const float* max_q, const float* denom, float threshold, int qblk, int batch, int heads,
+                                  int seq, int D, int kv_len, float scale, int max_blocks, void* stream);
+
 /* Top-k mask generator (python/spattn/mask_utils.py:389-417, qk_topkmask_indices): per
  * q-block of `blocksz` rows the select_k keys c < kv_len (0 = seq) with the largest
  * (block mean of q / sqrt(D)) . k[c], every step rounded to bf16 as the reference's bf16 torch

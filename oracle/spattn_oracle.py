@@ -342,6 +342,78 @@ def block_lists_from_mask(mask, seq: int, *, kvblk: int = 64, max_blocks: int | 
     return idx, cnt, bm
 
 
+def block_row_max(q, k, *, kv_len: int | None = None, kvblk: int = 64):
+    """Raw score maximum of every query row over every key block: out[b,h,J,r] = max over the
+    keys c of block J with c < kv_len of q[r].k[c] (fp32), -inf for a block without such a key,
+    laid out [B,H,Sp/kvblk,Sp] with Sp = 128*ceil(S/128); rows r >= S are left at 0.
+    The per-block form of the row maximum of include/maxq_denom.cuh:182,203."""
+    q = np.asarray(q, np.float32)
+    k = np.asarray(k, np.float32)
+    B, H, S, D = q.shape
+    kv = S if kv_len is None else kv_len
+    sp = padded_len(S)
+    nb = sp // kvblk
+    out = np.zeros((B, H, nb, sp), np.float32)
+    for b in range(B):
+        for h in range(H):
+            s = q[b, h] @ k[b, h, :kv].T
+            for j in range(nb):
+                c0, c1 = j * kvblk, min(kv, (j + 1) * kvblk)
+                out[b, h, j, :S] = s[:, c0:c1].max(axis=1) if c1 > c0 else -np.inf
+    return out
+
+
+def block_mask_from_blockmax(blockmax, max_q, denom, thresh: float, seq: int, D: int, *, qblk: int = 128,
+                             kv_len: int | None = None, scale: float | None = None, kvblk: int = 64):
+    """Block mask of the threshold test from per-(row, key block) score maxima:
+    MB[I,J] = OR_{r in q-block I, r < seq} blockmax[J][r] > t[r] with
+    t[r] = (log2 thresh + max_q[r] sf + log2 denom[r]) / sf - the test
+    exp2((s - max_q) sf) / denom > thresh of include/mask_utils.cuh:231-238 solved for s; some key
+    of a block passes it exactly when the block's maximum does.  Rows without a key (denom <= 0)
+    do not vote.  Returns (MB bool [B,H,ceil(S/qblk),Sp/kvblk], margin fp32 of the same shape:
+    max over the rows of (blockmax - t) sf, the log2 distance from the threshold)."""
+    bm = np.asarray(blockmax, np.float32)
+    B, H, nb, sp = bm.shape
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    sf = np.float32(LOG2E * scale)
+    kv = seq if kv_len is None else kv_len
+    nkb = ceil_div(kv, kvblk)
+    mx = np.asarray(max_q, np.float32).reshape(B, H, -1)[..., :seq]
+    dn = np.asarray(denom, np.float32).reshape(B, H, -1)[..., :seq]
+    with np.errstate(divide="ignore", invalid="ignore"):
+        t = np.where(dn > 0, (np.float32(np.log2(thresh)) + (mx * sf + np.log2(dn))) / sf, np.inf).astype(np.float32)
+    nq = ceil_div(seq, qblk)
+    mb = np.zeros((B, H, nq, nb), bool)
+    margin = np.full((B, H, nq, nb), -np.inf, np.float32)
+    for i in range(nq):
+        r0, r1 = i * qblk, min(seq, (i + 1) * qblk)
+        with np.errstate(invalid="ignore"):
+            d = (bm[:, :, :nkb, r0:r1] - t[:, :, None, r0:r1]) * sf      # [B,H,nkb,rows]
+        d = np.where(np.isnan(d), -np.inf, d)
+        margin[:, :, i, :nkb] = d.max(axis=-1)
+        mb[:, :, i, :nkb] = (bm[:, :, :nkb, r0:r1] > t[:, :, None, r0:r1]).any(axis=-1)
+    return mb, margin
+
+
+def block_lists_from_blockmask(bm, *, max_blocks: int | None = None, fill: int = -1):
+    """Ascending kept-block ids per row of a block mask [B,H,SB,NB], then `fill`; counts."""
+    bm = np.asarray(bm, bool)
+    B, H, SB, nb = bm.shape
+    if max_blocks is None:
+        max_blocks = nb
+    idx = np.full((B, H, SB, max_blocks), fill, np.int32)
+    cnt = np.zeros((B, H, SB), np.int32)
+    for b in range(B):
+        for h in range(H):
+            for i in range(SB):
+                nz = np.flatnonzero(bm[b, h, i])
+                cnt[b, h, i] = nz.size
+                w = min(nz.size, max_blocks)
+                idx[b, h, i, :w] = nz[:w]
+    return idx, cnt
+
+
 def pack_mask(mask):
     """Bit-packed form of a vote mask: bit (c & 7) of byte c >> 3 is set where mask[..., c] > 0
     (python/spattn/mask_utils.py:421-430, `pack`: 8 booleans per byte, least significant bit first).

@@ -256,6 +256,97 @@ def test_block_threshold_pipeline_feeds_block_attention(dev, qblk, D, S):
     assert_close_stat(f32(lse), wlse, "block pipeline lse")
 
 
+@pytest.mark.parametrize("with_v", [False, True])
+@pytest.mark.parametrize("D,S,kv_len", [(64, 1000, 0), (128, 700, 0), (64, 520, 450), (128, 64, 0), (64, 130, 1)])
+def test_block_maxima_of_the_statistics_sweeps(dev, D, S, kv_len, with_v):
+    """The statistics sweeps with the blockmax output: max_q / denom (and O) are bit for bit those of
+    the plain sweeps, blockmax[J][r] is the oracle's per-block row maximum, and its maximum over
+    the blocks is max_q exactly."""
+    print("case blockmax sweep", D, S, kv_len, with_v, flush=True)
+    B, H = 1, 3
+    q, k, v = wl.clustered_qkv(B, H, S, D, seed=71, sigma=0.7)
+    qd, kd, vd = to_dev(dev, q, k, v)
+    kv = kv_len or S
+    Sp = orc.padded_len(S)
+    nb, nkb = Sp // 64, orc.ceil_div(kv, 64)
+    mx, dn, mx2, dn2 = (torch.full((B, H, 1, Sp), 7.0, device=dev) for _ in range(4))
+    bmx = torch.full((B, H, nb, Sp), 123.0, device=dev)
+    if with_v:
+        o, o2 = torch.full_like(qd, float("nan")), torch.full_like(qd, float("nan"))
+        capi.fullattn_maxq_denom(o, mx, dn, qd, kd, vd, kv_len=kv_len)
+        capi.fullattn_maxq_denom_blockmax(o2, mx2, dn2, bmx, qd, kd, vd, kv_len=kv_len)
+        assert torch.equal(o.view(torch.int16), o2.view(torch.int16))
+    else:
+        capi.maxq_denom(mx, dn, qd, kd, kv_len=kv_len)
+        capi.maxq_denom_blockmax(mx2, dn2, bmx, qd, kd, kv_len=kv_len)
+    assert torch.equal(mx, mx2) and torch.equal(dn, dn2)
+    got = bmx.cpu().numpy()
+    want = orc.block_row_max(f32(q), f32(k), kv_len=kv)
+    assert np.all(got[:, :, nkb:] == 123.0), "blocks without a key are not written"
+    g, w = got[:, :, :nkb, :S], want[:, :, :nkb, :S]
+    assert np.isfinite(g).all() and np.isfinite(w).all()
+    assert np.all(np.abs(g - w) <= 1e-3 + 1e-4 * np.abs(w)), "blockmax differs from the oracle: %g" % np.abs(g - w).max()
+    assert np.array_equal(g.max(axis=2), mx.cpu().numpy().reshape(B, H, Sp)[..., :S])
+
+
+@pytest.mark.parametrize("qblk", [64, 128])
+@pytest.mark.parametrize("D,S,kv_len", [(64, 1000, 0), (128, 700, 0), (64, 520, 450), (64, 130, 1)])
+def test_block_lists_from_block_maxima(dev, qblk, D, S, kv_len):
+    """blockmax_to_blocklists: lists, counts and block mask are exactly the threshold of the device's
+    own block maxima and statistics (outside a thin band where the device's log2 may round the
+    other way), they agree with the block mask of the per-key oracle outside the threshold band,
+    and with the bit-packed sweep of the same threshold wherever the oracle is clear."""
+    print("case blockmax lists", qblk, D, S, kv_len, flush=True)
+    B, H = 1, 3
+    q, k, v = wl.clustered_qkv(B, H, S, D, seed=73, sigma=0.7)
+    qd, kd = to_dev(dev, q, k)
+    kv = kv_len or S
+    Sp = orc.padded_len(S)
+    nb, nkb, nq = Sp // 64, orc.ceil_div(kv, 64), orc.ceil_div(S, qblk)
+    mx = torch.empty((B, H, 1, Sp), device=dev)
+    dn = torch.empty((B, H, 1, Sp), device=dev)
+    bmx = torch.full((B, H, nb, Sp), float("nan"), device=dev)
+    capi.maxq_denom_blockmax(mx, dn, bmx, qd, kd, kv_len=kv_len)
+    _, pmax = orc.booleanmask_rows(f32(mx), f32(dn), f32(q), f32(k), 1.0, qblk=qblk, kv_len=kv)
+    pblk = np.full((B, H, nq, nb), -np.inf, np.float32)
+    for J in range(nkb):
+        pblk[..., J] = pmax[..., 64 * J: min(64 * J + 64, kv)].max(axis=-1)
+    # about 40 % of the blocks pass; with one or two blocks per row, a threshold every row passes
+    thr = float(np.quantile(pblk[..., :nkb], 0.6)) if nkb > 2 else 0.5 * float(pblk[..., :nkb].min())
+    bi = torch.full((B, H, nq, nb), -1, dtype=torch.int32, device=dev)
+    bc = torch.full((B, H, nq), -9, dtype=torch.int32, device=dev)
+    bm = torch.full((B, H, nq, nb), 7, dtype=torch.uint8, device=dev)
+    capi.blockmax_to_blocklists(bi, bc, bmx, mx, dn, thr, S, D, qblk=qblk, blockmask=bm, kv_len=kv_len)
+    got_bm = bm.cpu().numpy().astype(bool)
+    assert set(np.unique(bm.cpu().numpy())) <= {0, 1} and not got_bm[..., nkb:].any()
+    # the lists are the block mask, ascending, exact counts, fill behind them
+    wi, wn = orc.block_lists_from_blockmask(got_bm, fill=-1)
+    assert np.array_equal(bi.cpu().numpy(), wi) and np.array_equal(bc.cpu().numpy(), wn)
+    # the block mask is the threshold of the device's block maxima
+    dev_bmx = np.nan_to_num(bmx.cpu().numpy(), nan=-np.inf)
+    want_bm, margin = orc.block_mask_from_blockmax(dev_bmx, f32(mx), f32(dn), thr, S, D, qblk=qblk, kv_len=kv)
+    near = np.abs(margin) <= 1e-4
+    assert np.array_equal(got_bm | near, want_bm | near) and near.mean() < 0.01
+    # ... and the block mask of the per-key threshold mask, outside the band
+    band = np.abs(pblk - thr) <= BAND * thr
+    assert np.array_equal(got_bm | band, (pblk > np.float32(thr)) | band)
+    if nkb > 2:
+        assert 0.1 < got_bm[..., :nkb].mean() < 0.9
+    # the bit-packed sweep -> block lists route gives the same blocks where the oracle is clear
+    pk = torch.empty((B, H, nq, Sp // 8), dtype=torch.uint8, device=dev)
+    capi.booleanmask_packed(pk, mx, dn, qd, kd, thr, qblk=qblk, kv_len=kv_len)
+    bi2 = torch.full((B, H, nq, nb), -1, dtype=torch.int32, device=dev)
+    bc2 = torch.zeros((B, H, nq), dtype=torch.int32, device=dev)
+    bm2 = torch.zeros((B, H, nq, nb), dtype=torch.uint8, device=dev)
+    capi.packedmask_to_blocklists(bi2, bc2, pk, kv, blockmask=bm2)
+    assert np.array_equal(got_bm | band, bm2.cpu().numpy().astype(bool) | band)
+    # a list cut off at max_blocks keeps the first ids and the full count
+    bi3 = torch.full((B, H, nq, 2), -1, dtype=torch.int32, device=dev)
+    bc3 = torch.zeros((B, H, nq), dtype=torch.int32, device=dev)
+    capi.blockmax_to_blocklists(bi3, bc3, bmx, mx, dn, thr, S, D, qblk=qblk, kv_len=kv_len)
+    assert torch.equal(bc3, bc) and torch.equal(bi3, bi[..., :2])
+
+
 def test_all_index_mask(dev):
     print("case all_index_mask", flush=True)
     B, H, SB, S, ms = 2, 3, 5, 600, 640

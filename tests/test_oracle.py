@@ -266,6 +266,61 @@ def test_block_mask_and_block_lists_by_brute_force():
             assert set(ki[0, h, i, : kn[0, h, i]]) <= set(tok[0, h, i, : num[0, h, i]])
 
 
+def test_block_row_max_and_its_threshold_by_brute_force():
+    """blockmax[J][r] = max of the raw scores of row r over the keys of block J below kv_len
+    (plain loops), and thresholding it per row gives the block mask of the per-key threshold mask:
+    a key of block J passes softmax(r, c) > tau exactly when the block's maximum passes
+    s > t[r] - checked against block_mask_from_votes(booleanmask_rows(...)) outside a thin band
+    around the threshold, and exactly in float64."""
+    rng = np.random.default_rng(5)
+    B, H, S, D, kv = 1, 2, 520, 64, 450
+    q = orc.bf16_round(rng.standard_normal((B, H, S, D), dtype=np.float32))
+    k = orc.bf16_round(rng.standard_normal((B, H, S, D), dtype=np.float32) + np.repeat(
+        1.2 * rng.standard_normal((B, H, 13, D), dtype=np.float32), 40, axis=2))
+    bmx = orc.block_row_max(q, k, kv_len=kv)
+    sp = orc.padded_len(S)
+    assert bmx.shape == (B, H, sp // 64, sp)
+    for h in range(H):
+        for r in (0, 17, 199):
+            for J in range(sp // 64):
+                cols = range(64 * J, min(64 * J + 64, kv))
+                want = max((float(np.dot(q[0, h, r].astype(np.float64), k[0, h, c].astype(np.float64))) for c in cols),
+                           default=-np.inf)
+                assert bmx[0, h, J, r] == pytest.approx(want, rel=1e-5, abs=1e-5) or (want == -np.inf and bmx[0, h, J, r] == -np.inf)
+    assert np.all(bmx[..., S:] == 0) and np.all(bmx[:, :, 8:, :S] == -np.inf)   # blocks 8.. hold no key below 450
+    mx, dn = orc.maxq_denom(q, k, kv_len=kv)
+    for qblk in (64, 128):
+        mask, pmax = orc.booleanmask_rows(mx, dn, q, k, 1.0, qblk=qblk, kv_len=kv)
+        thr = float(np.quantile(pmax, 0.985))
+        want = orc.block_mask_from_votes((pmax > np.float32(thr)).astype(np.int32), kv)
+        got, margin = orc.block_mask_from_blockmax(bmx, mx, dn, thr, S, D, qblk=qblk, kv_len=kv)
+        nkb = orc.ceil_div(kv, 64)
+        assert got.shape == (B, H, orc.ceil_div(S, qblk), sp // 64) and not got[..., nkb:].any()
+        near = np.abs(margin[..., :nkb]) <= 1e-4
+        assert np.array_equal(got[..., :nkb] | near, want | near)
+        assert 0.02 < want.mean() < 0.98 and near.mean() < 0.01
+        # the same statement in float64, where the two forms of the test are the same inequality
+        # up to one rounding: compare the margins' signs away from zero
+        s64 = np.einsum("bhrd,bhcd->bhrc", q.astype(np.float64), k[:, :, :kv].astype(np.float64))
+        sf = orc.LOG2E / np.sqrt(D)
+        mx64 = s64.max(-1); dn64 = np.exp2((s64 - mx64[..., None]) * sf).sum(-1)
+        p64 = np.exp2((s64 - mx64[..., None]) * sf) / dn64[..., None]
+        for i in range(orc.ceil_div(S, qblk)):
+            rows = slice(i * qblk, min(S, (i + 1) * qblk))
+            for J in range(nkb):
+                cols = slice(64 * J, min(64 * J + 64, kv))
+                by_key = (p64[:, :, rows, cols] > thr).any(axis=(-1, -2))
+                t64 = (np.log2(thr) + mx64[:, :, rows] * sf + np.log2(dn64[:, :, rows])) / sf
+                by_block = (s64[:, :, rows, cols].max(-1) > t64).any(-1)
+                assert np.array_equal(by_key, by_block)
+    idx, cnt = orc.block_lists_from_blockmask(got, max_blocks=3, fill=-2)
+    for h in range(H):
+        for i in range(got.shape[2]):
+            kept = np.flatnonzero(got[0, h, i]).tolist()
+            assert cnt[0, h, i] == len(kept) and idx[0, h, i, : min(3, len(kept))].tolist() == kept[:3]
+            assert np.all(idx[0, h, i, len(kept):] == -2)
+
+
 def test_all_index_mask():
     idx, num = orc.all_index_mask(1, 2, 3, 300, 384)
     assert idx.shape == (1, 2, 3, 384) and np.all(idx == np.arange(384)) and np.all(num == 300)
