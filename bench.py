@@ -317,6 +317,9 @@ def bench_cfg4_end_to_end(dev, steps, warmup, seed=0):
                 (the reference's own sequence)
       blocks128 bit-packed sweep -> block lists -> sp_attn_blocks, 128-row q-blocks
       blocks64  the same with a mask row and a list per 64 query rows
+      blockmax128 / blockmax64  one sweep: the statistics pass also writes per-(row, key block) score maxima,
+                whose threshold gives the block lists (prepass_plus_attention_ms counts what the extra output
+                costs the statistics sweep instead of a second sweep)
     Every attention launch uses the work order computed (untimed here, timed on its own) from its counts."""
     c = wl.CONFIGS["cfg4_threshold_padded"]
     B, H, S, D = c["B"], c["H"], c["S"], c["D"]
@@ -407,7 +410,61 @@ def bench_cfg4_end_to_end(dev, steps, warmup, seed=0):
             "sp_attn_blocks_ms": ms_at, "sp_attn_blocks_tflops": fl / ms_at / 1e9,
             "sp_attn_blocks_mfma_frac": fl / ms_at / 1e9 / PEAK_BF16_TFLOPS,
             "prepass_plus_attention_ms": ms_sw + ms_bl + ms_order + ms_at}
+    # routes 4 and 5: one sweep.  The statistics sweep also writes the score maximum of every row over
+    # every 64-key block (1.6 GB); the threshold test runs on those maxima - no second Q K^T sweep.
+    del pk
+    bmx = torch.empty((B, H, nb, Sp), dtype=torch.float32, device=dev)
+    ms_fb, _ = time_steps(lambda: capi.fullattn_maxq_denom_blockmax(o, mx, dn, bmx, q, k, v), n_sw, 1)
+    ms_mb, _ = time_steps(lambda: capi.maxq_denom_blockmax(mx, dn, bmx, q, k), n_sw, 1)
+    out["fullattn_maxq_denom_blockmax"] = {"ms": ms_fb, "blockmax_bytes": 4.0 * bmx.numel()}
+    out["maxq_denom_blockmax"] = {"ms": ms_mb, "blockmax_bytes": 4.0 * bmx.numel()}
+    for qblk in (128, 64):
+        nq = wl.ceil_div(S, qblk)
+        biq = torch.full((B, H, nq, nb), -1, dtype=torch.int32, device=dev)
+        bcq = torch.zeros((B, H, nq), dtype=torch.int32, device=dev)
+        ms_bl, _ = time_steps(lambda: capi.blockmax_to_blocklists(biq, bcq, bmx, mx, dn, tau, S, D, qblk=qblk), steps, warmup)
+        kept = int(bcq.sum().item())
+        ordq = torch.empty((bcq.numel(),), dtype=torch.int32, device=dev)
+        capi.qblock_order(ordq, bcq)
+        ms_at, _ = time_steps(lambda: capi.sp_attn_blocks(o, q, k, v, biq, bcq, qblk=qblk, order=ordq), n_at, 2)
+        fl = wl.kept_block_flops(kept, qblk, 64, D)
+        # maxima of the blocks that hold a key, the two statistics rows, lists and counts
+        bl_bytes = 4.0 * B * H * nkb * S + 8.0 * B * H * S + 4.0 * kept + 4.0 * bcq.numel()
+        out["blockmax%d" % qblk] = {
+            "blockmax_to_blocklists_ms": ms_bl, "blockmax_to_blocklists_gbps": bl_bytes / ms_bl / 1e6,
+            "blockmax_to_blocklists_hbm_frac": bl_bytes / ms_bl / 1e6 / PEAK_HBM_GBPS, "blockmax_to_blocklists_bytes": bl_bytes,
+            "kept_blocks": kept, "block_density": kept / (float(bcq.numel()) * nkb),
+            "sp_attn_blocks_ms": ms_at, "sp_attn_blocks_tflops": fl / ms_at / 1e9,
+            "sp_attn_blocks_mfma_frac": fl / ms_at / 1e9 / PEAK_BF16_TFLOPS,
+            "extra_sweep_ms": ms_mb - out["maxq_denom"]["ms"],
+            "prepass_plus_attention_ms": (ms_mb - out["maxq_denom"]["ms"]) + ms_bl + ms_order + ms_at}
     assert torch.isfinite(o.float()).all().item(), "non-finite attention output"
+    return out
+
+
+def bench_blockmax(dev, steps, warmup, seed=0, tau=0.0102):
+    """The block-level mask pass on its own at the cfg 4 shape: one statistics sweep with the
+    per-(row, key block) maxima (untimed), then blockmax_to_blocklists timed - the leg the
+    FETCH_SIZE / WRITE_SIZE passes of profiles/ run."""
+    c = wl.CONFIGS["cfg4_threshold_padded"]
+    B, H, S, D = c["B"], c["H"], c["S"], c["D"]
+    q, k, _ = (t.to(dev) for t in wl.clustered_qkv(B, H, S, D, seed=seed))
+    Sp = 128 * wl.ceil_div(S, 128)
+    nb, nkb = Sp // 64, wl.ceil_div(S, 64)
+    mx = torch.empty((B, H, 1, Sp), device=dev)
+    dn = torch.empty((B, H, 1, Sp), device=dev)
+    bmx = torch.empty((B, H, nb, Sp), dtype=torch.float32, device=dev)
+    capi.maxq_denom_blockmax(mx, dn, bmx, q, k)
+    out = {"workload": "cfg4 block maxima fp32 [1,24,512,32768], threshold %g" % tau}
+    for qblk in (128, 64):
+        nq = wl.ceil_div(S, qblk)
+        bi = torch.full((B, H, nq, nb), -1, dtype=torch.int32, device=dev)
+        bc = torch.zeros((B, H, nq), dtype=torch.int32, device=dev)
+        ms, _ = time_steps(lambda: capi.blockmax_to_blocklists(bi, bc, bmx, mx, dn, tau, S, D, qblk=qblk), steps, warmup)
+        kept = int(bc.sum().item())
+        nbytes = 4.0 * B * H * nkb * S + 8.0 * B * H * S + 4.0 * kept + 4.0 * bc.numel()
+        out["q%d" % qblk] = {"ms": ms, "bytes": nbytes, "gbps": nbytes / ms / 1e6, "hbm_frac": nbytes / ms / 1e6 / PEAK_HBM_GBPS,
+                             "kept_blocks": kept, "block_density": kept / (float(bc.numel()) * nkb)}
     return out
 
 
@@ -505,7 +562,7 @@ def main(argv=None) -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-extras", action="store_true", help="only the headline kernel")
-    ap.add_argument("--only", default="", help="run one leg only: sparse|tokens|compact|dense|sweeps|copy|packed|topk|zipf|zipf64|cfg4|ldsprobe|gemm (no JSON contract)")
+    ap.add_argument("--only", default="", help="run one leg only: sparse|tokens|compact|dense|sweeps|copy|packed|topk|zipf|zipf64|cfg4|ldsprobe|gemm|blockmax (no JSON contract)")
     args = ap.parse_args(argv)
     if args.gpus != 1:
         print("bench.py: this library is single-GPU; run with --gpus 1 (got %d)" % args.gpus, file=sys.stderr)
@@ -520,7 +577,7 @@ def main(argv=None) -> int:
     if args.only:
         fn = {"sparse": bench_sparse, "compact": bench_compaction, "dense": bench_dense, "sweeps": bench_sweeps,
               "copy": bench_copy, "packed": bench_packed, "tokens": bench_tokens, "topk": bench_topk, "zipf": bench_zipf,
-              "zipf64": bench_zipf_sparse, "cfg4": bench_cfg4_end_to_end, "ldsprobe": bench_lds_probe, "gemm": bench_gemm}[args.only]
+              "zipf64": bench_zipf_sparse, "cfg4": bench_cfg4_end_to_end, "ldsprobe": bench_lds_probe, "gemm": bench_gemm, "blockmax": bench_blockmax}[args.only]
         r = fn(dev, args.steps, args.warmup)
         r.pop("tensors", None)
         r.pop("step", None)
@@ -581,6 +638,15 @@ def main(argv=None) -> int:
                                          "unit": "GB/s", "frac": tk4["booleanmask_to_indexmask_hbm_frac"],
                                          "traffic": measured_traffic("compact_kernel"), "traffic_unit": "bytes",
                                          "algorithmic_bytes": tk4["booleanmask_to_indexmask_bytes"]}}
+        bm4 = e2e["blockmax128"]
+        out["mask_pass_block"] = {"kernel": "blockmax_to_blocklists_kernel<128> (threshold of the per-(row, key block) score maxima -> block lists)",
+                                  "workload": "cfg4 block maxima fp32 [1, 24, 512, 32768] of the statistics sweep, %.1f%% of the blocks kept"
+                                              % (100.0 * bm4["block_density"]),
+                                  "ms": bm4["blockmax_to_blocklists_ms"],
+                                  "roofline": {"bound": "hbm", "achieved": bm4["blockmax_to_blocklists_gbps"], "peak": PEAK_HBM_GBPS,
+                                               "unit": "GB/s", "frac": bm4["blockmax_to_blocklists_hbm_frac"],
+                                               "traffic": measured_traffic("blockmax_to_blocklists_kernel<128>"), "traffic_unit": "bytes",
+                                               "algorithmic_bytes": bm4["blockmax_to_blocklists_bytes"]}}
         pk = e2e.pop("mask_cache")
         out["mask_cache"] = {
             "workload": "same mask, bit-packed (1 bit per key)",

@@ -251,6 +251,81 @@ void maxq_denom(torch::Tensor o_max_q, torch::Tensor o_denom, torch::Tensor q, t
   maxq_denom_ex(o_max_q, o_denom, q, k, 0.0, 0);
 }
 
+// The statistics sweeps with the per-(row, key block) score maxima as a further output, and the
+// threshold test on those maxima: the block-level form of booleanmask_128 + booleanmask_to_indexmask
+// (python/extension.cpp:229-340) that needs no second sweep over Q K^T.
+void check_blockmax(const torch::Tensor& blockmax, const torch::Tensor& q_like, int64_t B, int64_t H, int64_t S) {
+  check_aux(blockmax, "blockmax", at::kFloat, q_like);
+  const int64_t sp = padded128(S);
+  TORCH_CHECK(blockmax.numel() == B * H * (sp / 64) * sp, "blockmax must be fp32 [B,H,Sp/64,Sp] with Sp = 128*ceil(S/128)");
+}
+
+void fullattn_maxq_denom_blockmax(torch::Tensor o, torch::Tensor o_max_q, torch::Tensor o_denom, torch::Tensor blockmax,
+                                  torch::Tensor q, torch::Tensor k, torch::Tensor v, double scale, int64_t kv_len) {
+  check_bhsd(q, "q", q);
+  check_bhsd(k, "k", q);
+  check_bhsd(v, "v", q);
+  check_bhsd(o, "o", q);
+  check_aux(o_max_q, "o_max_q", at::kFloat, q);
+  check_aux(o_denom, "o_denom", at::kFloat, q);
+  const int64_t need = q.size(0) * q.size(1) * padded128(q.size(2));
+  TORCH_CHECK(o_max_q.numel() == need && o_denom.numel() == need, "o_max_q / o_denom must be [B,H,1,128*ceil(S/128)]");
+  check_blockmax(blockmax, q, q.size(0), q.size(1), q.size(2));
+  const DeviceGuard guard(q.device());
+  check_status(spattn_fullattn_maxq_denom_blockmax(o.data_ptr(), o_max_q.data_ptr<float>(), o_denom.data_ptr<float>(),
+                                                   blockmax.data_ptr<float>(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                                   (int)q.size(0), (int)q.size(1), (int)q.size(2), (int)q.size(3),
+                                                   checked_kv_len(kv_len, q), (float)scale, cur_stream()),
+               "fullattn_maxq_denom_blockmax");
+}
+
+void maxq_denom_blockmax(torch::Tensor o_max_q, torch::Tensor o_denom, torch::Tensor blockmax, torch::Tensor q,
+                         torch::Tensor k, double scale, int64_t kv_len) {
+  check_bhsd(q, "q", q);
+  check_bhsd(k, "k", q);
+  check_aux(o_max_q, "o_max_q", at::kFloat, q);
+  check_aux(o_denom, "o_denom", at::kFloat, q);
+  const int64_t need = q.size(0) * q.size(1) * padded128(q.size(2));
+  TORCH_CHECK(o_max_q.numel() == need && o_denom.numel() == need, "o_max_q / o_denom must be [B,H,1,128*ceil(S/128)]");
+  check_blockmax(blockmax, q, q.size(0), q.size(1), q.size(2));
+  const DeviceGuard guard(q.device());
+  check_status(spattn_maxq_denom_blockmax(o_max_q.data_ptr<float>(), o_denom.data_ptr<float>(), blockmax.data_ptr<float>(),
+                                          q.data_ptr(), k.data_ptr(), (int)q.size(0), (int)q.size(1), (int)q.size(2),
+                                          (int)q.size(3), checked_kv_len(kv_len, q), (float)scale, cur_stream()),
+               "maxq_denom_blockmax");
+}
+
+// blk_idx int32 [B,H,ceil(seq/qblk),max_blocks], blk_cnt int32 with B*H*ceil(seq/qblk) entries,
+// blockmask optional uint8 [B,H,ceil(seq/qblk),Sp/64]; head_dim fixes the default scale (scale = 0).
+void blockmax_to_blocklists(torch::Tensor blk_idx, torch::Tensor blk_cnt, OptTensor blockmask, torch::Tensor blockmax,
+                            torch::Tensor o_max_q, torch::Tensor o_denom, double threshold, int64_t seq, int64_t head_dim,
+                            int64_t qblk, double scale, int64_t kv_len) {
+  TORCH_CHECK(blk_idx.is_cuda() && blk_idx.scalar_type() == at::kInt && blk_idx.is_contiguous() && blk_idx.dim() == 4,
+              "blk_idx must be a contiguous int32 device tensor [B,H,ceil(seq/qblk),max_blocks]");
+  TORCH_CHECK(qblk == 64 || qblk == 128, "qblk must be 64 or 128");
+  TORCH_CHECK(seq > 0 && kv_len >= 0 && kv_len <= seq, "seq must be positive and kv_len lie in [0, seq]");
+  const int64_t B = blk_idx.size(0), H = blk_idx.size(1), SB = blk_idx.size(2), sp = padded128(seq);
+  TORCH_CHECK(SB == (seq + qblk - 1) / qblk, "blk_idx must hold ceil(seq/qblk) lists per head");
+  check_aux(blk_cnt, "blk_cnt", at::kInt, blk_idx);
+  TORCH_CHECK(blk_cnt.numel() == B * H * SB, "blk_cnt must have B*H*ceil(seq/qblk) entries");
+  check_aux(o_max_q, "o_max_q", at::kFloat, blk_idx);
+  check_aux(o_denom, "o_denom", at::kFloat, blk_idx);
+  TORCH_CHECK(o_max_q.numel() == B * H * sp && o_denom.numel() == B * H * sp, "o_max_q / o_denom must be [B,H,1,128*ceil(S/128)]");
+  check_blockmax(blockmax, blk_idx, B, H, seq);
+  void* bm = nullptr;
+  if (blockmask.has_value() && blockmask->defined()) {
+    check_aux(*blockmask, "blockmask", at::kByte, blk_idx);
+    TORCH_CHECK(blockmask->numel() == B * H * SB * (sp / 64), "blockmask must be uint8 [B,H,ceil(seq/qblk),Sp/64]");
+    bm = blockmask->data_ptr();
+  }
+  const DeviceGuard guard(blk_idx.device());
+  check_status(spattn_blockmax_to_blocklists(blk_idx.data_ptr<int>(), blk_cnt.data_ptr<int>(), bm, blockmax.data_ptr<float>(),
+                                             o_max_q.data_ptr<float>(), o_denom.data_ptr<float>(), (float)threshold, (int)qblk,
+                                             (int)B, (int)H, (int)seq, (int)head_dim, (int)kv_len, (float)scale,
+                                             (int)blk_idx.size(3), cur_stream()),
+               "blockmax_to_blocklists");
+}
+
 void booleanmask_128_ex(torch::Tensor booleanmask, torch::Tensor o_max_q, torch::Tensor o_denom, torch::Tensor q,
                         torch::Tensor k, double threshold, double scale, int64_t kv_len) {
   check_bhsd(q, "q", q);
@@ -446,6 +521,11 @@ void noop_mask_ex(torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, to
 void noop_mask_packed(torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, double, int64_t, double,
                       int64_t) {}
 void noop_blocklists(torch::Tensor, torch::Tensor, OptTensor, torch::Tensor, int64_t) {}
+void noop_fmd_bm(torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, double,
+                 int64_t) {}
+void noop_md_bm(torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, double, int64_t) {}
+void noop_bm_lists(torch::Tensor, torch::Tensor, OptTensor, torch::Tensor, torch::Tensor, torch::Tensor, double, int64_t, int64_t,
+                   int64_t, double, int64_t) {}
 
 TORCH_LIBRARY_FRAGMENT(cuda_attn, m) {
   m.def("full_attn(Tensor(a!) o, Tensor q, Tensor k, Tensor v) -> ()");
@@ -469,6 +549,9 @@ TORCH_LIBRARY_FRAGMENT(cuda_attn, m) {
   m.def("packedmask_to_blocklists(Tensor(a!) blk_idx, Tensor(b!) blk_cnt, Tensor(c!)? blockmask, Tensor packed, int seq) -> ()");
   m.def("booleanmask_to_blocklists(Tensor(a!) blk_idx, Tensor(b!) blk_cnt, Tensor(c!)? blockmask, Tensor booleanmask, int seq) -> ()");
   m.def("qblock_order(Tensor(a!) order, Tensor counts) -> ()");
+  m.def("fullattn_maxq_denom_blockmax(Tensor(a!) o, Tensor(b!) o_max_q, Tensor(c!) o_denom, Tensor(d!) blockmax, Tensor q, Tensor k, Tensor v, float scale, int kv_len) -> ()");
+  m.def("maxq_denom_blockmax(Tensor(a!) o_max_q, Tensor(b!) o_denom, Tensor(c!) blockmax, Tensor q, Tensor k, float scale, int kv_len) -> ()");
+  m.def("blockmax_to_blocklists(Tensor(a!) blk_idx, Tensor(b!) blk_cnt, Tensor(c!)? blockmask, Tensor blockmax, Tensor o_max_q, Tensor o_denom, float threshold, int seq, int head_dim, int qblk, float scale, int kv_len) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(cuda_attn, Meta, m) {
@@ -492,6 +575,9 @@ TORCH_LIBRARY_IMPL(cuda_attn, Meta, m) {
   m.impl("packedmask_to_blocklists", noop_blocklists);
   m.impl("booleanmask_to_blocklists", noop_blocklists);
   m.impl("qblock_order", noop2);
+  m.impl("fullattn_maxq_denom_blockmax", noop_fmd_bm);
+  m.impl("maxq_denom_blockmax", noop_md_bm);
+  m.impl("blockmax_to_blocklists", noop_bm_lists);
 }
 
 // The CUDA dispatch key serves HIP tensors on PyTorch-ROCm.
@@ -516,6 +602,9 @@ TORCH_LIBRARY_IMPL(cuda_attn, CUDA, m) {
   m.impl("packedmask_to_blocklists", packedmask_to_blocklists);
   m.impl("booleanmask_to_blocklists", booleanmask_to_blocklists);
   m.impl("qblock_order", qblock_order);
+  m.impl("fullattn_maxq_denom_blockmax", fullattn_maxq_denom_blockmax);
+  m.impl("maxq_denom_blockmax", maxq_denom_blockmax);
+  m.impl("blockmax_to_blocklists", blockmax_to_blocklists);
 }
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -539,4 +628,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("packedmask_to_blocklists", &packedmask_to_blocklists, "bit-packed mask -> KV-block lists");
   m.def("booleanmask_to_blocklists", &booleanmask_to_blocklists, "vote mask -> KV-block lists");
   m.def("qblock_order", &qblock_order, "work order, longest list first");
+  m.def("fullattn_maxq_denom_blockmax", &fullattn_maxq_denom_blockmax, "fullattn_maxq_denom + per-block row maxima");
+  m.def("maxq_denom_blockmax", &maxq_denom_blockmax, "maxq_denom + per-block row maxima");
+  m.def("blockmax_to_blocklists", &blockmax_to_blocklists, "block maxima -> KV-block lists");
 }

@@ -342,6 +342,39 @@ def qk_blocklists_cuda(q, k, thresh, qblk=128, kv_len=0):
     return qk_blocklists_from_maxq_denom_cuda(max_q, denom, q, k, thresh, qblk, kv_len)
 
 
+def blockmax_buffer(q):
+    """fp32 [B,H,Sp/64,Sp] for the per-(row, key block) score maxima of a statistics sweep."""
+    B, H, S, _ = q.shape
+    sp = _padded(S)
+    return torch.empty((B, H, sp // KVBLK, sp), dtype=torch.float32, device=q.device)
+
+
+def blockmax_to_blocklists_cuda(blockmax, max_q, denom, thresh, seq, head_dim, qblk=128, kv_len=0, max_blocks=None,
+                                with_blockmask=False):
+    """Threshold test on the block maxima -> KV-block lists (padded with -1), counts and, optionally,
+    the block mask uint8 [B,H,ceil(S/qblk),Sp/64].  A new threshold needs no new sweep."""
+    B, H, nb, _ = blockmax.shape
+    nq = (seq + qblk - 1) // qblk
+    if max_blocks is None:
+        max_blocks = nb
+    blk_idx = torch.full((B, H, nq, max_blocks), -1, dtype=torch.int32, device=blockmax.device)
+    blk_cnt = torch.zeros((B, H, nq), dtype=torch.int32, device=blockmax.device)
+    blockmask = torch.empty((B, H, nq, nb), dtype=torch.uint8, device=blockmax.device) if with_blockmask else None
+    spattn_interface.blockmax_to_blocklists(blk_idx, blk_cnt, blockmask, blockmax, max_q.contiguous(), denom.contiguous(),
+                                            thresh, seq, head_dim, qblk, 0.0, kv_len)
+    return (blk_idx, blk_cnt, blockmask) if with_blockmask else (blk_idx, blk_cnt)
+
+
+def qk_blocklists_onepass_cuda(q, k, thresh, qblk=128, kv_len=0):
+    """KV-block lists from ONE sweep over Q K^T: the statistics sweep also writes the maximum of
+    every row over every 64-key block, and the threshold test runs on those maxima.  Same lists as
+    qk_blocklists_cuda except where a block's best key sits within rounding of the threshold."""
+    max_q, denom = _stats_buffers(q)
+    blockmax = blockmax_buffer(q)
+    spattn_interface.maxq_denom_blockmax(max_q, denom, blockmax, q.contiguous(), k.contiguous(), 0.0, kv_len)
+    return blockmax_to_blocklists_cuda(blockmax, max_q, denom, thresh, q.shape[2], q.shape[3], qblk, kv_len)
+
+
 def qk_blocklists(q, k, thresh=0.001, qblk=128):
     """Pure-torch definition of the block lists: block J of q-block I is kept when some row of I
     and some key of J have softmax > thresh.  Returns (blk_idx padded with -1, blk_cnt, blockmask)."""

@@ -109,15 +109,26 @@ def cached_attn_cuda(query, key, value, current_layer, ditrun, *args, **kwargs):
 
 def blockcached_attn_cuda(query, key, value, current_layer, ditrun, *args, **kwargs):
     """cached_attn_cuda at the granularity of 64-key blocks (no counterpart in the reference):
-    on the refresh steps dense attention with statistics, then the bit-packed threshold sweep and
-    the block lists for q-blocks of ``qblk`` rows (64 or 128, default 128), kept in a
+    on the refresh steps dense attention with statistics and per-block score maxima, whose threshold
+    gives the block lists for q-blocks of ``qblk`` rows (64 or 128, default 128) without a second
+    sweep (``onepass=False``: the bit-packed threshold sweep instead), kept in a
     ``mask_utils.BlockListCache``; on every other step ``sp_attn_block`` over the cached lists in
     their cached work order - one launch."""
     mask_cache = kwargs["mask_cache"]
     qblk = kwargs.get("qblk", 128)
     if mask_cache.run_fullattn(ditrun):
-        out, max_q, denom = _dense_with_stats(query, key, value)
-        blk_idx, blk_cnt = mask_utils.qk_blocklists_from_maxq_denom_cuda(max_q, denom, query, key, kwargs["thresh"], qblk)
+        if kwargs.get("onepass", True):
+            # the dense pass also writes the per-(row, key block) score maxima: the lists come from
+            # thresholding those, without a second sweep over Q K^T
+            out = _out_like(query)
+            max_q, denom = mask_utils._stats_buffers(query)
+            blockmax = mask_utils.blockmax_buffer(query)
+            spattn_interface.fullattn_maxq_denom_blockmax(out, max_q, denom, blockmax, *_c(query, key, value), 0.0, 0)
+            blk_idx, blk_cnt = mask_utils.blockmax_to_blocklists_cuda(blockmax, max_q, denom, kwargs["thresh"], query.shape[2],
+                                                                    query.shape[3], qblk)
+        else:
+            out, max_q, denom = _dense_with_stats(query, key, value)
+            blk_idx, blk_cnt = mask_utils.qk_blocklists_from_maxq_denom_cuda(max_q, denom, query, key, kwargs["thresh"], qblk)
         mask_cache.update_cache(current_layer, blk_idx, blk_cnt)
         return out
     blk_idx, blk_cnt = mask_cache.get_mask_from_cache(current_layer)

@@ -333,3 +333,88 @@ def test_cfg4_padded_threshold_pipeline(dev):
         s = f32(q[0, h, r]) @ kf[0, h, lst].T
         pp, den, _ = orc._softmax_rows(s, 0.125, True)
         assert_close_o(f32(o[0, h, r]), (pp @ vf[0, h, lst]) / den[:, None], "cfg4 sparse rows (%d,%d)" % (h, i))
+
+
+def test_cfg4_block_maxima_route(dev):
+    """cfg 4 at its size through the one-sweep block route: maxq_denom with the per-(row, key
+    block) maxima (1.6 GB), their threshold into block masks and lists for 128- and 64-row
+    q-blocks (6144 / 12288 rows, every one compared with the same test done by torch on the
+    device's own maxima), density, agreement with the per-key oracle on sampled q-blocks, and
+    block-list attention over the result."""
+    print("case cfg4 block maxima", flush=True)
+    c = wl.CONFIGS["cfg4_threshold_padded"]
+    B, H, S, D = c["B"], c["H"], c["S"], c["D"]
+    q, k, v = wl.clustered_qkv(B, H, S, D, seed=7)
+    qd, kd, vd = to_dev(dev, q, k, v)
+    Sp, nb = 32768, 512
+    sf = np.float32(orc.LOG2E / 8.0)
+    mx, dn, mx0, dn0 = (torch.empty((B, H, 1, Sp), device=dev) for _ in range(4))
+    bmx = torch.full((B, H, nb, Sp), float("nan"), device=dev)
+    capi.maxq_denom(mx0, dn0, qd, kd)
+    capi.maxq_denom_blockmax(mx, dn, bmx, qd, kd)
+    assert torch.equal(mx, mx0) and torch.equal(dn, dn0)
+    del mx0, dn0
+    assert torch.isfinite(bmx[..., :S]).all()
+    assert torch.equal(bmx[..., :S].max(dim=2).values, mx.view(B, H, Sp)[..., :S])
+    kf = f32(k)
+    rng = np.random.default_rng(8)
+    blocks = [(int(rng.integers(H)), int(rng.integers(256))) for _ in range(4)] + [(0, 255), (H - 1, 255)]
+    samp = []
+    for h, i in blocks + [(h, i) for h in (0, 11, 23) for i in range(0, 256, 32)]:
+        r = slice(i * 128, min(S, (i + 1) * 128))
+        s = f32(q[0, h, r]) @ kf[0, h].T
+        sb = np.concatenate([s, np.full((s.shape[0], Sp - S), -np.inf, np.float32)], axis=1).reshape(s.shape[0], nb, 64).max(-1)
+        got = bmx[0, h, :, r].cpu().numpy().T
+        assert np.all(np.abs(got - sb) <= 1e-3 + 1e-4 * np.abs(sb)), "blockmax (%d,%d)" % (h, i)
+        p = np.exp2((s - f32(mx)[0, h, 0, r, None]) * sf) / f32(dn)[0, h, 0, r, None]
+        samp.append(np.concatenate([p.max(0), np.zeros(Sp - S, np.float32)]).reshape(-1, 64).max(1))
+    thr = float(np.quantile(np.concatenate(samp[len(blocks):]), 0.92))
+    # what the threshold of the maxima must give, by torch on the device's own numbers
+    t = (np.float32(np.log2(thr)) + (mx.view(B, H, Sp) * float(sf) + torch.log2(dn.view(B, H, Sp)))) / float(sf)
+    t[..., S:] = float("inf")
+    margin = (bmx - t[:, :, None, :]) * float(sf)
+    margin[..., S:] = float("-inf")
+    lists = {}
+    for qblk in (128, 64):
+        nq = orc.ceil_div(S, qblk)
+        mg = margin.view(B, H, nb, Sp // qblk, qblk)[:, :, :, :nq]
+        want = (mg > 0).any(-1).transpose(2, 3)
+        near = (mg.abs() <= 1e-4).any(-1).transpose(2, 3)
+        bi = torch.full((B, H, nq, nb), -1, dtype=torch.int32, device=dev)
+        bc = torch.full((B, H, nq), -3, dtype=torch.int32, device=dev)
+        bm = torch.full((B, H, nq, nb), 9, dtype=torch.uint8, device=dev)
+        capi.blockmax_to_blocklists(bi, bc, bmx, mx, dn, thr, S, D, qblk=qblk, blockmask=bm)
+        assert int(bm.max()) <= 1
+        got = bm.bool()
+        assert torch.equal(got | near, want | near) and float(near.float().mean()) < 1e-3
+        assert torch.equal(bc, got.sum(-1).int())
+        ar = torch.arange(nb, device=dev, dtype=torch.int32)
+        want_bi = torch.where(got, ar, torch.full_like(ar, 1 << 20)).sort(-1).values
+        assert torch.equal(bi, torch.where(want_bi == (1 << 20), torch.full_like(want_bi, -1), want_bi))
+        lists[qblk] = (bi, bc, got)
+        del mg, want, near, bm, want_bi
+    del margin, t
+    dens = float(lists[128][2].float().mean())
+    assert 0.06 < dens < 0.10, dens
+    assert 0.03 < float(lists[64][2].float().mean()) < dens
+    # the per-key oracle on the sampled q-blocks, outside the threshold band
+    for (h, i), pb in zip(blocks, samp):
+        band = np.abs(pb - thr) <= 1e-2 * thr
+        assert np.array_equal(lists[128][2][0, h, i].cpu().numpy() | band, (pb > thr) | band), "block row (%d,%d)" % (h, i)
+    vf = f32(v)
+    for qblk in (128, 64):
+        bi, bc, _ = lists[qblk]
+        o = torch.full_like(qd, float("nan"))
+        capi.sp_attn_blocks(o, qd, kd, vd, bi, bc, qblk=qblk)
+        assert torch.isfinite(o.float()).all()
+        bih, bch = bi.cpu().numpy(), bc.cpu().numpy()
+        for h, i in blocks[:3] + blocks[-1:]:
+            j = i * (128 // qblk)
+            r = slice(j * qblk, min(S, (j + 1) * qblk))
+            tok, num = orc.block_list_to_token_list(bih[:, h:h + 1, j:j + 1], bch[:, h:h + 1, j:j + 1], S)
+            lst = tok[0, 0, 0, : num[0, 0, 0]]
+            if lst.size == 0:
+                assert not f32(o[0, h, r]).any()
+                continue
+            pp, den, _ = orc._softmax_rows(f32(q[0, h, r]) @ kf[0, h, lst].T, 0.125, True)
+            assert_close_o(f32(o[0, h, r]), (pp @ vf[0, h, lst]) / den[:, None], "cfg4 blockmax route q%d (%d,%d)" % (qblk, h, j))

@@ -228,6 +228,51 @@ def test_extended_operators_on_device(dev):
         ops.booleanmask_packed(packed, mx, dn, q, k, thr, 32, 0.0, 0)
 
 
+def test_block_maxima_operators_and_helpers(dev):
+    """torch.ops.cuda_attn.maxq_denom_blockmax / fullattn_maxq_denom_blockmax / blockmax_to_blocklists
+    against the C ABI (bit for bit), and the one-sweep helper against the two-sweep one: the same
+    block lists except where a block's best key lies within the band around the threshold."""
+    print("case blockmax operators", flush=True)
+    from fgattn_tk_cuda_amd.spattn import mask_utils as mu
+
+    ops = torch.ops.cuda_attn
+    B, H, S, D, thr = 1, 2, 900, 64, 0.01
+    q, k, v = to_dev(dev, *wl.clustered_qkv(B, H, S, D, seed=83, sigma=0.7))
+    Sp = orc.padded_len(S)
+    mx, dn, mx2, dn2 = (torch.empty((B, H, 1, Sp), device=dev) for _ in range(4))
+    bmx, bmx2 = (torch.full((B, H, Sp // 64, Sp), -5.0, device=dev) for _ in range(2))
+    o, o2 = torch.empty_like(q), torch.empty_like(q)
+    ops.fullattn_maxq_denom_blockmax(o, mx, dn, bmx, q, k, v, 0.0, 0)
+    capi.fullattn_maxq_denom_blockmax(o2, mx2, dn2, bmx2, q, k, v)
+    assert torch.equal(o, o2) and torch.equal(mx, mx2) and torch.equal(dn, dn2) and torch.equal(bmx, bmx2)
+    bmx3 = torch.full_like(bmx, -5.0)
+    ops.maxq_denom_blockmax(mx2, dn2, bmx3, q, k, 0.0, 0)
+    assert torch.equal(mx, mx2) and torch.equal(dn, dn2) and torch.equal(bmx, bmx3)
+    for qblk in (64, 128):
+        nq, nb = orc.ceil_div(S, qblk), Sp // 64
+        bi, bc, bm = mu.blockmax_to_blocklists_cuda(bmx, mx, dn, thr, S, D, qblk, with_blockmask=True)
+        bi2 = torch.full((B, H, nq, nb), -1, dtype=torch.int32, device=dev)
+        bc2 = torch.zeros((B, H, nq), dtype=torch.int32, device=dev)
+        capi.blockmax_to_blocklists(bi2, bc2, bmx, mx, dn, thr, S, D, qblk=qblk)
+        assert torch.equal(bi, bi2) and torch.equal(bc, bc2) and torch.equal(bm.sum(-1).int(), bc)
+        b1, c1 = mu.qk_blocklists_onepass_cuda(q, k, thr, qblk)
+        assert torch.equal(b1, bi) and torch.equal(c1, bc)
+        # two sweeps (bit-packed threshold sweep) against one: equal outside the band
+        _, _, bm_two = mu.packedmask_to_blocklists_cuda(mu.qk_packedmask_from_maxq_denom_cuda(mx, dn, q, k, thr, qblk), S,
+                                                        with_blockmask=True)
+        _, pmax = orc.booleanmask_rows(f32(mx), f32(dn), f32(q), f32(k), 1.0, qblk=qblk)
+        pblk = np.zeros((B, H, nq, nb), np.float32)
+        for J in range(orc.ceil_div(S, 64)):
+            pblk[..., J] = pmax[..., 64 * J: min(64 * J + 64, S)].max(axis=-1)
+        band = np.abs(pblk - thr) <= 1e-2 * thr
+        assert np.array_equal(bm.cpu().numpy().astype(bool) | band, bm_two.cpu().numpy().astype(bool) | band)
+        assert 0.05 < bm.float().mean().item() < 0.95
+    with pytest.raises(RuntimeError):
+        ops.blockmax_to_blocklists(bi, bc, None, bmx[:, :, :3].contiguous(), mx, dn, thr, S, D, 128, 0.0, 0)
+    with pytest.raises(RuntimeError):
+        ops.blockmax_to_blocklists(bi, bc, None, bmx, mx, dn, thr, S, D, 32, 0.0, 0)
+
+
 def test_functionals_with_mask_cache(dev):
     print("case functionals", flush=True)
     from fgattn_tk_cuda_amd.spattn import mask_utils as mu, sparseattn_functionals as fn
@@ -248,9 +293,9 @@ def test_functionals_with_mask_cache(dev):
         assert 0 < kvn.float().mean().item() < S
         if isinstance(cache, mu.NaiveMaskCache):
             assert cache.get_order(7) is not None and cache.get_order(7).numel() == kvn.numel()
-    for qblk in (64, 128):
+    for qblk, onepass in ((64, True), (128, True), (64, False), (128, False)):
         cache = mu.BlockListCache([0])
-        o0 = fn.blockcached_attn_cuda(q, k, v, 7, 0, thresh=0.01, qblk=qblk, mask_cache=cache)
+        o0 = fn.blockcached_attn_cuda(q, k, v, 7, 0, thresh=0.01, qblk=qblk, mask_cache=cache, onepass=onepass)
         assert_close_o(f32(o0), f32(dense), "block cache fill step")
         o1 = fn.blockcached_attn_cuda(q, k, v, 7, 1, thresh=0.01, qblk=qblk, mask_cache=cache)
         bi, bc = cache.get_mask_from_cache(7)
