@@ -57,21 +57,32 @@ def _run(cmd: list[str]) -> None:
         print(out)
 
 
-def build_lib(verbose: bool = True) -> Path:
-    """Compile every HIP translation unit and link libspattn_hip.so."""
-    OBJ.mkdir(exist_ok=True)
+POISON_LIB = PKG / "libspattn_hip_poison.so"
+
+
+def build_lib(verbose: bool = True, poison: bool = False) -> Path:
+    """Compile every HIP translation unit and link libspattn_hip.so.
+
+    poison=True builds libspattn_hip_poison.so instead: the same library with -DSPATTN_POISON_RING,
+    whose attention kernels fill every ring slot with NaNs between the barrier that frees it and the
+    copy that refills it (a debug build for the copy pipeline; tests compare it bit for bit with
+    the product library)."""
+    objdir = CSRC / ("_obj_poison" if poison else "_obj")
+    objdir.mkdir(exist_ok=True)
     hipcc = _hipcc()
+    flags = HIPCC_FLAGS + (["-DSPATTN_POISON_RING"] if poison else [])
     jobs = []
     for src in HIP_SOURCES:
-        obj = OBJ / (src.replace(".hip", ".o"))
-        jobs.append([hipcc, *HIPCC_FLAGS, "-c", str(CSRC / src), "-o", str(obj)])
+        obj = objdir / (src.replace(".hip", ".o"))
+        jobs.append([hipcc, *flags, "-c", str(CSRC / src), "-o", str(obj)])
     with ThreadPoolExecutor(max_workers=min(8, len(jobs))) as pool:
         list(pool.map(_run, jobs))
-    objs = [str(OBJ / s.replace(".hip", ".o")) for s in HIP_SOURCES]
-    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB), *objs])
+    objs = [str(objdir / s.replace(".hip", ".o")) for s in HIP_SOURCES]
+    out = POISON_LIB if poison else LIB
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(out), *objs])
     if verbose:
-        print("built", LIB)
-    return LIB
+        print("built", out)
+    return out
 
 
 PROBES = PKG / "libspattn_probes.so"
@@ -127,6 +138,7 @@ def main(argv=None) -> int:
     if not args.lib_only:
         build_torch_ext()
         build_probes()
+        build_lib(poison=True)
     return 0
 
 

@@ -689,6 +689,24 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     using GK = std::integral_constant<int, (KC + NK) % 3>;    // tile it+NK
     using GV = std::integral_constant<int, (KC + 1) % 3>;     // tile it+1
     const TileLoad tl_first = K_FIRST ? prepare_tile(d_k, KN, false, GK{}) : prepare_tile(d_v, VN, true, GV{});
+#ifdef SPATTN_POISON_RING
+    // Debug build of the copy pipeline: the two ring slots this barrier has freed are filled with
+    // bf16 NaNs before the copies of V(it+1) and K(it+NK) are issued into them (each wave the
+    // parts it copies itself, the stores complete before the copies go out).  A wave that still
+    // reads the old tile from a freed slot - a missing wait, a barrier too few, a wrong slot
+    // number - then sees NaNs instead of stale but plausible keys, and the output shows it.
+    {
+      const u32x4 nan4 = {0x7fc07fc0u, 0x7fc07fc0u, 0x7fc07fc0u, 0x7fc07fc0u};
+      auto poison = [&](int slot) {
+        unsigned char* base = smem + slot * TILE + wave * 1024 + lane * 16;
+#pragma unroll
+        for (int i = 0; i < LPT; ++i) *reinterpret_cast<u32x4*>(base + i * 4096) = nan4;
+      };
+      if constexpr (HAS_V) poison(VN);
+      if (has_kn) poison(KN);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    }
+#endif
     constexpr int PAR = KC & 1;
     qk_tile(std::true_type{}, std::integral_constant<bool, HAS_V>{}, KS * TILE, VS * TILE, s_b, s_a, PAR, &tl_first,
             K_FIRST ? has_kn : true);
