@@ -102,18 +102,16 @@ def board_state():
 
 def under_load(fn, ms_per_call: float, samples: int = 3):
     """Reads power and clock `samples` times while fn() runs back to back (untimed): each reading
-    is taken with about 1.5 s of launches already queued, so the GPU is busy while rocm-smi looks.
+    is taken right behind about one second of launches (the board's metrics lag by that much).
     The part runs this library's attention kernels at or near its power cap, and the clock it
     settles at, not the nominal 2.4 GHz, is what the matrix units get."""
     got = []
-    batch = max(8, min(20000, int(1500.0 / max(ms_per_call, 1e-3))))
-    for _ in range(batch // 2):
-        fn()
+    batch = max(8, min(20000, int(1000.0 / max(ms_per_call, 1e-3))))
     for _ in range(samples):
         for _ in range(batch):
             fn()
-        st = board_state()
         torch.cuda.synchronize()
+        st = board_state()
         if st is None:
             return None
         got.append(st)
@@ -607,8 +605,8 @@ def main(argv=None) -> int:
         out["board"] = {"during_sp_attn": board, "during_gemm": gm["board"],
                         "gemm_bf16_8192_tflops": gm["tflops"], "gemm_mfma_frac": gm["tflops"] / PEAK_BF16_TFLOPS,
                         "sp_attn_vs_gemm": tflops / gm["tflops"],
-                        "note": "rocm-smi socket power and graphics clock, averaged over samples taken while the "
-                                "kernel runs back to back; torch.mm (hipBLASLt) bf16 8192^3 timed like every leg"}
+                        "note": "rocm-smi socket power and graphics clock, three readings each taken right behind a second "
+                                "of back-to-back launches; torch.mm (hipBLASLt) bf16 8192^3 timed like every leg"}
         tk = bench_tokens(dev, args.steps, args.warmup, res=res)
         out["token_lists"] = {"workload": "cfg3 with the kept keys as token-id lists (the reference operator's form)",
                               "kernel": "attn_fwd_kernel<128,64,KV_TOKENS>", "ms": tk["ms"],
