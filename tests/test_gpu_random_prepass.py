@@ -153,3 +153,62 @@ def test_topk_generator_random(dev, seed):
     assert np.all(kvn == kk)
     assert np.array_equal(kvi[..., :kk], want_sel)
     assert np.all(kvi[..., kk:] == fill)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_block_maxima_route_random(dev, seed):
+    """The one-sweep block route on drawn shapes (from one query row and one key up): block maxima
+    against the oracle, their maximum over the blocks equal to max_q, the thresholded block mask
+    against the threshold of the device's own maxima and against the per-key oracle outside the
+    band, lists = the mask, for both q-block sizes."""
+    rng = np.random.default_rng(9000 + seed)
+    B, H = int(rng.integers(1, 3)), int(rng.integers(1, 4))
+    S = int(rng.choice([1, 31, 64, 65, 127, 129, 200, 333, 512, 641, 900]))
+    D = int(rng.choice([64, 128]))
+    kv_len = int(rng.choice([0, S, int(rng.integers(1, S + 1))]))
+    kv = kv_len or S
+    with_v = bool(rng.integers(2))
+    print("case random blockmax", seed, B, H, S, D, kv_len, with_v, flush=True)
+    q, k, v = wl.clustered_qkv(B, H, S, D, seed=seed, sigma=0.8)
+    qd, kd, vd = to_dev(dev, q, k, v)
+    Sp = orc.padded_len(S)
+    nb, nkb = Sp // 64, orc.ceil_div(kv, 64)
+    mx = torch.full((B, H, 1, Sp), float("nan"), device=dev)
+    dn = torch.full((B, H, 1, Sp), float("nan"), device=dev)
+    bmx = torch.full((B, H, nb, Sp), float("nan"), device=dev)
+    if with_v:
+        o = torch.full_like(qd, float("nan"))
+        capi.fullattn_maxq_denom_blockmax(o, mx, dn, bmx, qd, kd, vd, kv_len=kv_len)
+        want = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float()[:, :, :kv], v.float()[:, :, :kv])
+        assert_close_o(f32(o), f32(want), "fullattn_maxq_denom_blockmax O")
+    else:
+        capi.maxq_denom_blockmax(mx, dn, bmx, qd, kd, kv_len=kv_len)
+    wmx, wdn = orc.maxq_denom(f32(q), f32(k), kv_len=kv)
+    assert_close_stat(f32(mx), wmx, "max_q", atol=1e-4)
+    assert_close_stat(f32(dn), wdn, "denom")
+    got = bmx.cpu().numpy()
+    assert np.isnan(got[:, :, nkb:]).all(), "blocks without a key are not written"
+    g, w = got[:, :, :nkb, :S], orc.block_row_max(f32(q), f32(k), kv_len=kv)[:, :, :nkb, :S]
+    assert np.isfinite(g).all() and np.all(np.abs(g - w) <= 1e-3 + 1e-4 * np.abs(w))
+    assert np.array_equal(g.max(axis=2), f32(mx).reshape(B, H, Sp)[..., :S])
+    dev_bmx = np.nan_to_num(got, nan=-np.inf)
+    for qblk in (64, 128):
+        nq = orc.ceil_div(S, qblk)
+        _, pmax = orc.booleanmask_rows(f32(mx), f32(dn), f32(q), f32(k), 1.0, qblk=qblk, kv_len=kv)
+        pblk = np.full((B, H, nq, nb), -np.inf, np.float32)
+        for J in range(nkb):
+            pblk[..., J] = pmax[..., 64 * J: min(64 * J + 64, kv)].max(axis=-1)
+        thr = float(np.quantile(pblk[..., :nkb], 0.5)) if nkb > 2 else 0.5 * float(pblk[..., :nkb].min())
+        bi = torch.full((B, H, nq, nb), -1, dtype=torch.int32, device=dev)
+        bc = torch.full((B, H, nq), -9, dtype=torch.int32, device=dev)
+        bm = torch.full((B, H, nq, nb), 7, dtype=torch.uint8, device=dev)
+        capi.blockmax_to_blocklists(bi, bc, bmx, mx, dn, thr, S, D, qblk=qblk, blockmask=bm, kv_len=kv_len)
+        got_bm = bm.cpu().numpy().astype(bool)
+        assert int(bm.max()) <= 1 and not got_bm[..., nkb:].any()
+        wi, wn = orc.block_lists_from_blockmask(got_bm, fill=-1)
+        assert np.array_equal(bi.cpu().numpy(), wi) and np.array_equal(bc.cpu().numpy(), wn)
+        want_bm, margin = orc.block_mask_from_blockmax(dev_bmx, f32(mx), f32(dn), thr, S, D, qblk=qblk, kv_len=kv)
+        near = np.abs(margin) <= 1e-4
+        assert np.array_equal(got_bm | near, want_bm | near)
+        band = np.abs(pblk - thr) <= BAND * thr
+        assert np.array_equal(got_bm | band, (pblk > np.float32(thr)) | band)
