@@ -418,3 +418,70 @@ def test_cfg4_block_maxima_route(dev):
                 continue
             pp, den, _ = orc._softmax_rows(f32(q[0, h, r]) @ kf[0, h, lst].T, 0.125, True)
             assert_close_o(f32(o[0, h, r]), (pp @ vf[0, h, lst]) / den[:, None], "cfg4 blockmax route q%d (%d,%d)" % (qblk, h, j))
+
+
+def test_reference_shape_75856_with_its_kv_length(dev):
+    """The largest shape the reference compiles, B=1 H=24 S=75856 d=128, with the kv length it
+    hard-codes for it (75856 - 245, python/cuda_attn.cu:28-31): dense attention, fused statistics,
+    the threshold pre-pass and sparse attention over its lists, sampled q-blocks against the
+    oracle.  Keys 75611.. must not contribute anywhere."""
+    print("case reference shape 75856", flush=True)
+    B, H, S, D, kv = 1, 24, 75856, 128, 75856 - 245
+    g = torch.Generator(device=dev).manual_seed(5)
+    q, k, v = (torch.randn((B, H, S, D), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16) for _ in range(3))
+    k[:, :, kv:] = 50.0      # keys behind the kv length would dominate every row if they were read
+    v[:, :, kv:] = -50.0
+    Sp, SB = orc.padded_len(S), orc.ceil_div(S, 128)
+    sf = np.float32(orc.LOG2E / np.sqrt(D))
+    o = torch.full_like(q, float("nan"))
+    lse = torch.full((B, H, S), float("nan"), device=dev)
+    capi.full_attn(o, q, k, v, lse=lse, kv_len=kv)
+    o2 = torch.full_like(q, float("nan"))
+    mx = torch.full((B, H, 1, Sp), float("nan"), device=dev)
+    dn = torch.full((B, H, 1, Sp), float("nan"), device=dev)
+    capi.fullattn_maxq_denom(o2, mx, dn, q, k, v, kv_len=kv)
+    assert torch.isfinite(o.float()).all() and torch.isfinite(o2.float()).all()
+    rng = np.random.default_rng(6)
+    blocks = [(int(rng.integers(H)), int(rng.integers(SB))) for _ in range(3)] + [(H - 1, SB - 1), (0, kv // 128)]
+    per = {}
+    for h, i in blocks:
+        r = slice(i * 128, min(S, (i + 1) * 128))
+        qh, kh, vh = f32(q[0, h, r]), f32(k[0, h, :kv]), f32(v[0, h, :kv])
+        s = qh @ kh.T
+        m = s.max(1)
+        p = np.exp2((s - m[:, None]) * sf)
+        d = p.sum(1)
+        want = (orc.bf16_round(p) @ vh) / d[:, None]
+        assert_close_o(f32(o[0, h, r]), want, "full_attn rows (%d,%d)" % (h, i))
+        assert_close_o(f32(o2[0, h, r]), want, "fullattn_maxq_denom rows (%d,%d)" % (h, i))
+        assert_close_stat(f32(lse[0, h, r]), (m * sf + np.log2(d)) * np.float32(np.log(2.0)), "lse", atol=1e-3)
+        assert_close_stat(f32(mx)[0, h, 0, r], m, "max_q", atol=1e-3)
+        assert_close_stat(f32(dn)[0, h, 0, r], d, "denom")
+        per[(h, i)] = (p / d[:, None]).max(0)
+    del o2
+    thr = float(np.quantile(np.concatenate(list(per.values())), 0.98))
+    mask = torch.zeros((B, H, SB, Sp), dtype=torch.int32, device=dev)
+    capi.booleanmask_128(mask, mx, dn, q, k, thr, kv_len=kv)
+    assert not bool(mask[..., kv:].any())
+    kvi = torch.full((B, H, SB, Sp), Sp, dtype=torch.int32, device=dev)
+    kvn = torch.zeros((B, H, SB), dtype=torch.int32, device=dev)
+    capi.booleanmask_to_indexmask(kvi, kvn, mask, kv)
+    assert torch.equal(kvn, (mask > 0).sum(-1).int()) and int(kvn.max()) <= kv
+    for (h, i), pmax in per.items():
+        near = np.abs(pmax - thr) <= 1e-2 * thr
+        got = mask[0, h, i, :kv].cpu().numpy() > 0
+        assert np.array_equal(got | near, (pmax > thr) | near), "mask row (%d,%d)" % (h, i)
+        n = int(kvn[0, h, i])
+        assert np.array_equal(kvi[0, h, i, :n].cpu().numpy(), np.flatnonzero(got))
+    del mask
+    o3 = torch.full_like(q, float("nan"))
+    capi.sp_attn(o3, q, k, v, kvi, kvn, kv_len=kv)
+    assert torch.isfinite(o3.float()).all()
+    for h, i in blocks:
+        r = slice(i * 128, min(S, (i + 1) * 128))
+        lst = kvi[0, h, i, : int(kvn[0, h, i])].cpu().numpy()
+        if lst.size == 0:
+            assert not f32(o3[0, h, r]).any()
+            continue
+        pp, den, _ = orc._softmax_rows(f32(q[0, h, r]) @ f32(k[0, h])[lst].T, 1.0 / np.sqrt(D), True)
+        assert_close_o(f32(o3[0, h, r]), (pp @ f32(v[0, h])[lst]) / den[:, None], "sp_attn rows (%d,%d)" % (h, i))
