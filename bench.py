@@ -602,6 +602,11 @@ def main(argv=None) -> int:
         # what the board does while the headline kernel runs, and what its library GEMM reaches
         board = under_load(res["step"], res["ms"])
         gm = bench_gemm(dev, max(2, args.steps // 4), 2)
+        if board and board.get("gfxclk_mhz"):
+            # the nominal peak is quoted at 2.4 GHz; under this kernel the board holds a lower clock
+            peak_at_clock = PEAK_BF16_TFLOPS * board["gfxclk_mhz"] / 2400.0
+            out["roofline"]["at_sustained_clock"] = {"gfxclk_mhz": board["gfxclk_mhz"], "peak": peak_at_clock,
+                                                     "frac": tflops / peak_at_clock}
         out["board"] = {"during_sp_attn": board, "during_gemm": gm["board"],
                         "gemm_bf16_8192_tflops": gm["tflops"], "gemm_mfma_frac": gm["tflops"] / PEAK_BF16_TFLOPS,
                         "sp_attn_vs_gemm": tflops / gm["tflops"],
