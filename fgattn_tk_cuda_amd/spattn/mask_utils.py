@@ -71,6 +71,33 @@ class OffloadMaskCache(NaiveMaskCache):
 
     def update_cache(self, layer, kv_indices, kv_num_indices):
         self.cache[layer] = (kv_indices.cpu(), kv_num_indices)
+        self.order[layer] = qblock_order_cuda(kv_num_indices) if _is_dev(kv_num_indices) else None
+
+
+class CompressMaskCache(NaiveMaskCache):
+    """The reference's compressed list cache (python/spattn/mask_utils.py:46-67) keeps the index
+    lists through nvcomp's BitComp codec.  Here the lists are kept as what they encode - one bit
+    per (q-block, key), 1/32 of the int32 lists - and come back through the fused
+    bits -> lists kernel: the same keys per q-block, in ascending order (the attention operators do
+    not depend on the order), with the fill value the reference uses (the row length)."""
+
+    def get_mask_from_cache(self, layer):
+        packed, seq_len, kv_num_indices = self.cache[layer]
+        kv_indices, counts = packedmask_to_indexmask_cuda(packed, seq_len)
+        return kv_indices, counts.view_as(kv_num_indices)
+
+    def update_cache(self, layer, kv_indices, kv_num_indices):
+        B, H, SB, stride = kv_indices.shape
+        pos = torch.arange(stride, device=kv_indices.device).view(1, 1, 1, stride)
+        live = (pos < kv_num_indices.reshape(B, H, SB, 1)) & (kv_indices >= 0) & (kv_indices < stride)
+        votes = torch.zeros((B, H, SB, stride + 1), dtype=torch.int32, device=kv_indices.device)
+        # entries behind the count (or outside the row) are sent to a spare column
+        votes.scatter_(3, torch.where(live, kv_indices, torch.full_like(kv_indices, stride)).long(), 1)
+        votes = votes[..., :stride].contiguous()
+        seq_len = int(stride)
+        packed = pack_votes_cuda(votes) if votes.is_cuda and stride % 128 == 0 else pack(votes > 0)
+        self.cache[layer] = (packed, seq_len, kv_num_indices)
+        self.order[layer] = qblock_order_cuda(kv_num_indices) if _is_dev(kv_num_indices) else None
 
 
 class BitMaskCache:

@@ -65,6 +65,13 @@ def attn_computed_with_sparse_mask_python(query, key, value, current_layer=None,
     return _sparse(query, key, value, kv_indices, kv_num_indices)
 
 
+def attn_lshmask_cuda(query, key, value, current_layer=None, ditrun=None, *args, **kwargs):
+    """LSH-selected key lists, then sparse attention (:51-58).  As in the reference the selector is
+    not implemented (python/spattn/mask_utils.py:385-386): the call raises NotImplementedError."""
+    kv_indices, kv_num_indices = mask_utils.qk_lshmask_indices(query, key, kwargs["thresh"], blocksz=kwargs["blocksz"])
+    return _sparse(query, key, value, kv_indices, kv_num_indices)
+
+
 def attn_topkmask_cuda(query, key, value, current_layer=None, ditrun=None, *args, **kwargs):
     """Top-k key lists per q-block, then sparse attention (:39-48).  The lists come from the
     device selector, padded to a multiple of 128 keys as the sparse operator needs."""

@@ -282,7 +282,10 @@ def test_functionals_with_mask_cache(dev):
     dense = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float())
     assert_close_o(f32(fn.baseline_attn(q, k, v, 0, 0)), f32(dense), "baseline_attn")
     assert_close_o(f32(fn.baseline_attn_maxq_denom(q, k, v, 0, 0)), f32(dense), "baseline_attn_maxq_denom")
-    for cache in (mu.NaiveMaskCache([0]), mu.BitMaskCache([0]), mu.CompressedBitMaskCache([0])):
+    with pytest.raises(NotImplementedError):
+        fn.attn_lshmask_cuda(q, k, v, 0, 0, thresh=0.01, blocksz=128)
+    for cache in (mu.NaiveMaskCache([0]), mu.CompressMaskCache([0]), mu.OffloadMaskCache([0]), mu.BitMaskCache([0]),
+                  mu.CompressedBitMaskCache([0])):
         f = fn.cached_attn_cuda if isinstance(cache, mu.NaiveMaskCache) else fn.bitmaskcached_attn_cuda
         o0 = f(q, k, v, 7, 0, thresh=0.01, blocksz=128, mask_cache=cache)       # step 0: dense + cache fill
         assert_close_o(f32(o0), f32(dense), "cache fill step")
@@ -293,6 +296,10 @@ def test_functionals_with_mask_cache(dev):
         assert 0 < kvn.float().mean().item() < S
         if isinstance(cache, mu.NaiveMaskCache):
             assert cache.get_order(7) is not None and cache.get_order(7).numel() == kvn.numel()
+        if isinstance(cache, mu.CompressMaskCache):
+            # the compressed cache returns the lists it was given (as sets per q-block; here ascending both ways)
+            ref_i, ref_n = mu.qk_indexmask_cuda(q, k, 0.01, blocksz=128)
+            assert torch.equal(kvn.view_as(ref_n), ref_n) and torch.equal(kvi, ref_i)
     for qblk, onepass in ((64, True), (128, True), (64, False), (128, False)):
         cache = mu.BlockListCache([0])
         o0 = fn.blockcached_attn_cuda(q, k, v, 7, 0, thresh=0.01, qblk=qblk, mask_cache=cache, onepass=onepass)
