@@ -46,6 +46,8 @@ _SIGNATURES = {
     "spattn_maxq_denom_blockmax": (_c_int, [_c_void_p] * 5 + [_c_int] * 5 + [_c_float, _c_void_p]),
     "spattn_fullattn_maxq_denom_blockmax": (_c_int, [_c_void_p] * 7 + [_c_int] * 5 + [_c_float, _c_void_p]),
     "spattn_blockmax_to_blocklists": (_c_int, [_c_void_p] * 6 + [_c_float] + [_c_int] * 6 + [_c_float, _c_int, _c_void_p]),
+    "spattn_booleanmask_128_blocks": (_c_int, [_c_void_p, _c_float, _c_int] + [_c_void_p] * 6 + [_c_int] * 6 + [_c_float, _c_void_p]),
+    "spattn_booleanmask_packed_blocks": (_c_int, [_c_void_p, _c_float, _c_int, _c_int] + [_c_void_p] * 6 + [_c_int] * 6 + [_c_float, _c_void_p]),
     "spattn_pack_mask": (_c_int, [_c_void_p] * 2 + [_c_int] * 4 + [_c_void_p]),
     "spattn_packedmask_to_indexmask": (_c_int, [_c_void_p] * 3 + [_c_int] * 5 + [_c_void_p]),
     "spattn_qk_topkmask_indices": (_c_int, [_c_void_p] * 6 + [_c_int] * 9 + [_c_void_p]),
@@ -247,6 +249,42 @@ def booleanmask_packed(packed, max_q, denom, q, k, threshold, *, qblk=128, kv_le
     _check(load().spattn_booleanmask_packed(_ptr(packed, torch.uint8), float(threshold), int(packed.shape[3]) * 8,
                                             int(qblk), _ptr(max_q, f32), _ptr(denom, f32), _ptr(q, bf16), _ptr(k, bf16),
                                             B, H, S, D, kv_len, scale, _stream(stream)))
+
+
+def _lists128(blk_indices, blk_counts, B, H, S):
+    SB = (S + 127) // 128
+    if blk_indices.dim() != 4 or tuple(blk_indices.shape[:3]) != (B, H, SB) or blk_counts.numel() != B * H * SB:
+        raise ValueError("blk_indices must be [B,H,ceil(S/128),max_blocks] and blk_counts hold B*H*ceil(S/128) entries")
+
+
+def booleanmask_128_blocks(booleanmask, max_q, denom, q, k, threshold, blk_indices, blk_counts, *, kv_len=0, scale=0.0,
+                           stream=None):
+    """booleanmask_128 restricted to the 64-key blocks listed per 128-row q-block; the rest of the mask is zeroed."""
+    B, H, S, D = _bhsd(q)
+    _need_padded(max_q, denom, B, H, S)
+    _lists128(blk_indices, blk_counts, B, H, S)
+    if booleanmask.dim() != 4 or int(booleanmask.shape[2]) != (S + 127) // 128:
+        raise ValueError("booleanmask must be [B,H,ceil(S/128),mask_stride]")
+    _check(load().spattn_booleanmask_128_blocks(_ptr(booleanmask, i32), float(threshold), int(booleanmask.shape[3]),
+                                                _ptr(max_q, f32), _ptr(denom, f32), _ptr(q, bf16), _ptr(k, bf16),
+                                                _ptr(blk_indices, i32), _ptr(blk_counts, i32), int(blk_indices.shape[3]),
+                                                B, H, S, D, kv_len, scale, _stream(stream)))
+
+
+def booleanmask_packed_blocks(packed, max_q, denom, q, k, threshold, blk_indices, blk_counts, *, qblk=128, kv_len=0,
+                              scale=0.0, stream=None):
+    """booleanmask_packed restricted to the listed blocks (lists per 128-row q-block for either qblk)."""
+    B, H, S, D = _bhsd(q)
+    _need_padded(max_q, denom, B, H, S)
+    _lists128(blk_indices, blk_counts, B, H, S)
+    if qblk not in (64, 128):
+        raise ValueError("qblk must be 64 or 128")
+    if packed.dim() != 4 or tuple(packed.shape[:3]) != (B, H, (S + qblk - 1) // qblk):
+        raise ValueError("packed must be uint8 [B,H,ceil(S/qblk),mask_stride/8]")
+    _check(load().spattn_booleanmask_packed_blocks(_ptr(packed, torch.uint8), float(threshold), int(packed.shape[3]) * 8,
+                                                   int(qblk), _ptr(max_q, f32), _ptr(denom, f32), _ptr(q, bf16),
+                                                   _ptr(k, bf16), _ptr(blk_indices, i32), _ptr(blk_counts, i32),
+                                                   int(blk_indices.shape[3]), B, H, S, D, kv_len, scale, _stream(stream)))
 
 
 def _blocklist_args(blk_indices, blk_counts, blockmask, B, H, SB, MS):

@@ -188,6 +188,40 @@ int spattn_booleanmask_packed(void* packed, float threshold, int mask_stride, in
                                           kv < mask_stride ? kv : mask_stride, sc, as_stream(stream)));
 }
 
+int spattn_booleanmask_128_blocks(int* booleanmask, float threshold, int mask_stride, const float* max_q, const float* denom,
+                                  const void* q, const void* k, const int* blk_indices, const int* blk_counts, int max_blocks,
+                                  int B, int H, int S, int D, int kv_len, float scale, void* stream) {
+  if (int st = check_qkv(q, k, B, H, S, D)) return done(st);
+  if (!booleanmask || !max_q || !denom || !blk_indices || !blk_counts) return done(SPATTN_ERR_NULL);
+  if (mask_stride <= 0 || mask_stride % 128 != 0) return done(SPATTN_ERR_STRIDE);
+  if (max_blocks <= 0) return done(SPATTN_ERR_SHAPE);
+  if (misaligned(booleanmask)) return done(SPATTN_ERR_ALIGN);
+  const int kv = (kv_len <= 0 || kv_len > S) ? S : kv_len;
+  const float sc = scale > 0.f ? scale : 1.0f / sqrtf((float)D);
+  return from_hip(spattn::run_booleanmask(booleanmask, 0, threshold, mask_stride, max_q, denom,
+                                          static_cast<const uint16_t*>(q), static_cast<const uint16_t*>(k), B, H, S, D,
+                                          kv < mask_stride ? kv : mask_stride, sc, as_stream(stream), blk_indices, blk_counts,
+                                          max_blocks));
+}
+
+int spattn_booleanmask_packed_blocks(void* packed, float threshold, int mask_stride, int qblk, const float* max_q,
+                                     const float* denom, const void* q, const void* k, const int* blk_indices,
+                                     const int* blk_counts, int max_blocks, int B, int H, int S, int D, int kv_len,
+                                     float scale, void* stream) {
+  if (int st = check_qkv(q, k, B, H, S, D)) return done(st);
+  if (!packed || !max_q || !denom || !blk_indices || !blk_counts) return done(SPATTN_ERR_NULL);
+  if (qblk != 64 && qblk != 128) return done(SPATTN_ERR_QBLK);
+  if (mask_stride <= 0 || mask_stride % 128 != 0) return done(SPATTN_ERR_STRIDE);
+  if (max_blocks <= 0) return done(SPATTN_ERR_SHAPE);
+  if (misaligned(packed)) return done(SPATTN_ERR_ALIGN);
+  const int kv = (kv_len <= 0 || kv_len > S) ? S : kv_len;
+  const float sc = scale > 0.f ? scale : 1.0f / sqrtf((float)D);
+  return from_hip(spattn::run_booleanmask(packed, qblk, threshold, mask_stride, max_q, denom,
+                                          static_cast<const uint16_t*>(q), static_cast<const uint16_t*>(k), B, H, S, D,
+                                          kv < mask_stride ? kv : mask_stride, sc, as_stream(stream), blk_indices, blk_counts,
+                                          max_blocks));
+}
+
 int spattn_packedmask_to_blocklists(int* blk_indices, int* blk_counts, void* blockmask, const void* packed, int B, int H,
                                     int seq, int seqblocks, int mask_stride, int max_blocks, void* stream) {
   if (!blk_indices || !blk_counts || !packed) return done(SPATTN_ERR_NULL);

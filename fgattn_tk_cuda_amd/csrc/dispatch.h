@@ -12,7 +12,8 @@ hipError_t run_attn_dense(const AttnParams& p, int D, bool has_v, bool stats, hi
 // mask_kernels.hip
 hipError_t run_booleanmask(void* out, int out_rows, float thresh, int mask_stride, const float* max_q,
                            const float* denom, const uint16_t* q, const uint16_t* k, int B, int H, int S, int D,
-                           int kv_len, float scale, hipStream_t stream);
+                           int kv_len, float scale, hipStream_t stream, const int* blk_idx = nullptr,
+                           const int* blk_cnt = nullptr, int max_blocks = 0);
 hipError_t run_compact(int* kv_indices, int* kv_num, const int* mask, int rows, int mask_stride, int kv_len,
                        hipStream_t stream);
 hipError_t run_all_index(int* kv_indices, int* kv_num, int rows, int mask_stride, int seq, hipStream_t stream);

@@ -42,13 +42,19 @@ namespace spattn {
 // ------------------------------------------------------------------------------------
 enum MaskOut : int { OUT_VOTES = 0, OUT_BITS128 = 1, OUT_BITS64 = 2 };
 
-template <int D, int OUT>
+// SPARSE: the sweep restricted to the 64-key blocks of a per-q-block list (ascending ids, e.g. the
+// block lists that the threshold of the block maxima gives): a key of a block whose maximum fails
+// the test cannot pass it, so every other entry of the mask row is zero and the multiplies of the
+// kept blocks give the same votes as the full sweep.  The workgroup first clears its mask row(s),
+// then each wave walks every fourth 32-key half block of the listed blocks.
+template <int D, int OUT, bool SPARSE>
 __global__ __launch_bounds__(256, 2) void booleanmask_kernel(int* __restrict__ mask, const float* __restrict__ max_q,
                                                               const float* __restrict__ denom,
                                                               const uint16_t* __restrict__ q,
                                                               const uint16_t* __restrict__ k, float log2_thresh,
                                                               int mask_stride, int HB, int S, int kv_len, int Sp,
-                                                              int SB, float sf) {
+                                                              int SB, float sf, const int* __restrict__ blk_idx,
+                                                              const int* __restrict__ blk_cnt, int max_blocks) {
   constexpr int NT = D / 16;
   constexpr int CPR = D / 8;
   constexpr bool Q_REGS = (D == 64);
@@ -128,6 +134,46 @@ __global__ __launch_bounds__(256, 2) void booleanmask_kernel(int* __restrict__ m
     if (2 * qb + 1 < nq64) brow1 = brow0 + nkb;
   }
 
+  // The walk of this workgroup: position j -> 32-key block.  Dense: block j.  Sparse: the two
+  // halves of the listed 64-key blocks in list order; positions before the first stand for "no
+  // block" (nothing is stored for them), positions past the last repeat the last one (their keys
+  // are copied, never multiplied), an id outside the row is replaced by the row's last block.
+  typedef const __attribute__((address_space(4))) int* cint_p;
+  cint_p lst = nullptr;
+  int nseq = nkb;
+  if constexpr (SPARSE) {
+    const size_t lrow = (size_t)bh * SB + qb;
+    int n = ((cint_p)blk_cnt)[lrow];
+    n = n < 0 ? 0 : (n > max_blocks ? max_blocks : n);
+    nseq = 2 * n;
+    lst = (cint_p)(blk_idx + lrow * max_blocks);
+    // clear the row(s): 16-byte stores, then every store of the workgroup has reached memory
+    // before any wave writes a vote
+    const i32x4 z4 = {0, 0, 0, 0};
+    if constexpr (OUT == OUT_VOTES) {
+      for (int i = tid * 4; i < mask_stride; i += 1024) *reinterpret_cast<i32x4*>(mrow + i) = z4;
+    } else {
+      for (int i = tid * 4; i < nkb; i += 1024) {
+        *reinterpret_cast<i32x4*>(brow0 + i) = z4;
+        if (OUT == OUT_BITS64 && brow1 != nullptr) *reinterpret_cast<i32x4*>(brow1 + i) = z4;
+      }
+    }
+    wait_vmcnt<0>();
+    __syncthreads();
+  }
+  auto kb_at = [&](int j) -> int {
+    if constexpr (!SPARSE) {
+      return j;
+    } else {
+      if (j < 0) return -1;
+      int jj = j < nseq ? j : nseq - 1;
+      jj = jj < 0 ? 0 : jj;
+      int e = nseq > 0 ? lst[jj >> 1] : 0;
+      e = (unsigned)e < (unsigned)(nkb >> 1) ? e : (nkb >> 1) - 1;
+      return 2 * e + (jj & 1);
+    }
+  };
+
   // Ring layout: key row r of a block at r * 2D bytes, its 16-byte chunk c at c ^ kswz(r),
   // which spreads chunk 2t+g of the 32 rows a half wave reads over all bank groups.  Copy i
   // of a block moves rows 8i .. 8i+7: lane l fills position l of that 1 KB, i.e. fetches the
@@ -155,6 +201,7 @@ __global__ __launch_bounds__(256, 2) void booleanmask_kernel(int* __restrict__ m
       for (int i = 0; i < 4; ++i) {
         int key = kb * 32 + krow[i];
         key = key < kv_len ? key : kv_len - 1;
+        key = key < 0 ? 0 : key;
         dma16(kh, (uint32_t)key * (D * 2) + kcol[i],
               __builtin_amdgcn_readfirstlane(ring_base + slot * KBLK + i * 1024));
       }
@@ -174,6 +221,7 @@ __global__ __launch_bounds__(256, 2) void booleanmask_kernel(int* __restrict__ m
   auto load_keys = [&](int kb, u32x4 (&kf)[NT]) {
     int key = kb * 32 + ln;
     key = key < kv_len ? key : kv_len - 1;
+    key = key < 0 ? 0 : key;
 #pragma unroll
     for (int t = 0; t < NT; ++t) kf[t] = *reinterpret_cast<const u32x4*>(kh + (size_t)key * D + 16 * t + 8 * g);
   };
@@ -251,9 +299,9 @@ __global__ __launch_bounds__(256, 2) void booleanmask_kernel(int* __restrict__ m
       }
     }
   };
-  // Half H: multiplies pair H&1 of block kb into acc[H % NACC] and reduces the accumulators
-  // of the half before.
-  auto half = [&](auto hc, int kb, u32x4 (&kf)[NT], bool reload, uint32_t next_lds) {
+  // Half H: multiplies pair H&1 of the current block into acc[H % NACC] and reduces the
+  // accumulators of the half before; kb_prev: the block before the current one in this wave's walk.
+  auto half = [&](auto hc, int kb_prev, u32x4 (&kf)[NT], bool reload, uint32_t next_lds) {
     constexpr int H = decltype(hc)::value;
     constexpr int P = H & 1, A = H % NACC, AP = (H + NACC - 1) % NACC;
     pair_scores(P, kf, acc[A], reload, next_lds);
@@ -264,7 +312,7 @@ __global__ __launch_bounds__(256, 2) void booleanmask_kernel(int* __restrict__ m
       __builtin_amdgcn_sched_group_barrier(0x002, (NT == 4) ? 3 : 2, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (P == 0) finish_block(kb - 4, vhold | v);   // pair 1 of the block before
+    if constexpr (P == 0) finish_block(kb_prev, vhold | v);   // pair 1 of the block before
     else vhold = v;                                          // pair 0 of this block
   };
   // After the last block (its second half went into acc[A]): reduce it and store.
@@ -275,7 +323,7 @@ __global__ __launch_bounds__(256, 2) void booleanmask_kernel(int* __restrict__ m
   using I0 = std::integral_constant<int, 0>;
   using I1 = std::integral_constant<int, 1>;
 
-  int kb = wave;
+  int j = wave;          // position in the walk; this wave takes every fourth
   acc[1][0] = nthr[2];   // reduced by the very first half; its votes go nowhere
   acc[1][1] = nthr[3];
   if constexpr (K_RING) {
@@ -285,39 +333,39 @@ __global__ __launch_bounds__(256, 2) void booleanmask_kernel(int* __restrict__ m
     // blocks b+2 and b+3 are always there (vote stores may or may not be), hence vmcnt(8).
     u32x4 kf[NT];
     int slot = 0;
-    issue_keys(kb, 0);
-    issue_keys(kb + 4, 1);
-    issue_keys(kb + 8, 2);
+    issue_keys(kb_at(j), 0);
+    issue_keys(kb_at(j + 4), 1);
+    issue_keys(kb_at(j + 8), 2);
     wait_vmcnt<8>();
     read_keys(0, kf);
-    auto block = [&](auto h0, auto h1, int kbb) {
-      issue_keys(kbb + 12, (slot + 3) & (NSLOT - 1));
-      half(h0, kbb, kf, false, 0u);
+    auto block = [&](auto h0, auto h1, int jj) {
+      issue_keys(kb_at(jj + 12), (slot + 3) & (NSLOT - 1));
+      half(h0, kb_at(jj - 4), kf, false, 0u);
       wait_vmcnt<8>();
-      half(h1, kbb, kf, true, slot_addr(slot + 1));
+      half(h1, 0, kf, true, slot_addr(slot + 1));
       slot = (slot + 1) & (NSLOT - 1);
     };
-    for (; kb < nkb; kb += 4) block(I0{}, I1{}, kb);
-    drain(I1{}, kb - 4);
+    for (; j < nseq; j += 4) block(I0{}, I1{}, j);
+    drain(I1{}, kb_at(j - 4));
     wait_vmcnt<0>();   // no copy may land after the workgroup has given up its LDS
   } else {
     u32x4 k0[NT], k1[NT];
-    load_keys(kb, k0);
-    while (kb + 4 < nkb) {
-      load_keys(kb + 4, k1);
-      half(I0{}, kb, k0, false, 0u);
-      half(I1{}, kb, k0, false, 0u);
-      load_keys(kb + 8, k0);
-      half(I0{}, kb + 4, k1, false, 0u);
-      half(I1{}, kb + 4, k1, false, 0u);
-      kb += 8;
+    load_keys(kb_at(j), k0);
+    while (j + 4 < nseq) {
+      load_keys(kb_at(j + 4), k1);
+      half(I0{}, kb_at(j - 4), k0, false, 0u);
+      half(I1{}, 0, k0, false, 0u);
+      load_keys(kb_at(j + 8), k0);
+      half(I0{}, kb_at(j), k1, false, 0u);
+      half(I1{}, 0, k1, false, 0u);
+      j += 8;
     }
-    if (kb < nkb) {
-      half(I0{}, kb, k0, false, 0u);
-      half(I1{}, kb, k0, false, 0u);
-      drain(I1{}, kb);
+    if (j < nseq) {
+      half(I0{}, kb_at(j - 4), k0, false, 0u);
+      half(I1{}, 0, k0, false, 0u);
+      drain(I1{}, kb_at(j));
     } else {
-      drain(I1{}, kb - 4);
+      drain(I1{}, kb_at(j - 4));
     }
   }
 }
@@ -325,15 +373,22 @@ __global__ __launch_bounds__(256, 2) void booleanmask_kernel(int* __restrict__ m
 template <int D, int OUT>
 static void launch_booleanmask(int* mask, float lt, int mask_stride, const float* max_q, const float* denom,
                                const uint16_t* q, const uint16_t* k, int HB, int S, int kv_len, int Sp, int SB, float sf,
-                               hipStream_t stream) {
-  hipLaunchKernelGGL((booleanmask_kernel<D, OUT>), dim3(SB * HB, 1, 1), dim3(256), 0, stream, mask, max_q, denom, q, k,
-                     lt, mask_stride, HB, S, kv_len, Sp, SB, sf);
+                               const int* blk_idx, const int* blk_cnt, int max_blocks, hipStream_t stream) {
+  if (blk_idx != nullptr)
+    hipLaunchKernelGGL((booleanmask_kernel<D, OUT, true>), dim3(SB * HB, 1, 1), dim3(256), 0, stream, mask, max_q, denom, q,
+                       k, lt, mask_stride, HB, S, kv_len, Sp, SB, sf, blk_idx, blk_cnt, max_blocks);
+  else
+    hipLaunchKernelGGL((booleanmask_kernel<D, OUT, false>), dim3(SB * HB, 1, 1), dim3(256), 0, stream, mask, max_q, denom, q,
+                       k, lt, mask_stride, HB, S, kv_len, Sp, SB, sf, nullptr, nullptr, 0);
 }
 
 // out_rows: 0 = int32 vote counts; 128 / 64 = bit rows per q-block of that many query rows.
+// blk_idx / blk_cnt / max_blocks: optional lists of 64-key blocks per 128-row q-block
+// ([B,H,SB,max_blocks] ascending ids, [B,H,SB] counts) that restrict the sweep (see SPARSE above).
 hipError_t run_booleanmask(void* out, int out_rows, float thresh, int mask_stride, const float* max_q,
                            const float* denom, const uint16_t* q, const uint16_t* k, int B, int H, int S, int D,
-                           int kv_len, float scale, hipStream_t stream) {
+                           int kv_len, float scale, hipStream_t stream, const int* blk_idx, const int* blk_cnt,
+                           int max_blocks) {
   const int SB = (S + 127) / 128;
   const int Sp = SB * 128;
   const float sf = kLog2e * scale;
@@ -342,7 +397,8 @@ hipError_t run_booleanmask(void* out, int out_rows, float thresh, int mask_strid
   if (total <= 0) return hipSuccess;
   int* m = static_cast<int*>(out);
   const int HB = H * B;
-#define SPATTN_MASK_CASE(DD, OO) launch_booleanmask<DD, OO>(m, lt, mask_stride, max_q, denom, q, k, HB, S, kv_len, Sp, SB, sf, stream)
+#define SPATTN_MASK_CASE(DD, OO) \
+  launch_booleanmask<DD, OO>(m, lt, mask_stride, max_q, denom, q, k, HB, S, kv_len, Sp, SB, sf, blk_idx, blk_cnt, max_blocks, stream)
   if (D == 128) {
     if (out_rows == 0) SPATTN_MASK_CASE(128, OUT_VOTES);
     else if (out_rows == 128) SPATTN_MASK_CASE(128, OUT_BITS128);

@@ -181,6 +181,26 @@ int spattn_blockmax_to_blocklists(int* blk_indices, int* blk_counts, void* block
                                   const float* max_q, const float* denom, float threshold, int qblk, int batch, int heads,
                                   int seq, int D, int kv_len, float scale, int max_blocks, void* stream);
 
+/* The threshold sweep restricted to listed key blocks.  blk_indices int32
+ * [batch,heads,ceil(seq/128),max_blocks] holds, per 128-row q-block, ascending ids of 64-key
+ * blocks, blk_counts [batch,heads,ceil(seq/128)] how many.  Only the keys of the listed blocks are
+ * multiplied and tested; every other entry of the mask row is written as zero.  With lists that
+ * hold every block in which some key passes the test - what spattn_blockmax_to_blocklists gives at
+ * qblk = 128 for the same statistics, threshold, scale and kv_len - the result is the mask of
+ * spattn_booleanmask_128 / spattn_booleanmask_packed (include/mask_utils.cuh:131-243), vote for
+ * vote, at the cost of the kept blocks only (about 8 % of the sweep at the density the reference
+ * runs at).  A block missing from a list loses its votes; an id outside the row is ignored.
+ * booleanmask / packed, mask_stride, qblk as in the full sweeps (qblk is the row granularity of
+ * the bit output; the lists are per 128-row q-block in both cases). */
+int spattn_booleanmask_128_blocks(int* booleanmask, float threshold, int mask_stride, const float* max_q,
+                                  const float* denom, const void* q, const void* k, const int* blk_indices,
+                                  const int* blk_counts, int max_blocks, int batch, int heads, int seq, int D, int kv_len,
+                                  float scale, void* stream);
+int spattn_booleanmask_packed_blocks(void* packed, float threshold, int mask_stride, int qblk, const float* max_q,
+                                     const float* denom, const void* q, const void* k, const int* blk_indices,
+                                     const int* blk_counts, int max_blocks, int batch, int heads, int seq, int D,
+                                     int kv_len, float scale, void* stream);
+
 /* Top-k mask generator (python/spattn/mask_utils.py:389-417, qk_topkmask_indices): per
  * q-block of `blocksz` rows the select_k keys c < kv_len (0 = seq) with the largest
  * (block mean of q / sqrt(D)) . k[c], every step rounded to bf16 as the reference's bf16 torch

@@ -347,6 +347,79 @@ def test_block_lists_from_block_maxima(dev, qblk, D, S, kv_len):
     assert torch.equal(bc3, bc) and torch.equal(bi3, bi[..., :2])
 
 
+@pytest.mark.parametrize("D,S,kv_len", [(64, 1000, 0), (128, 700, 0), (64, 520, 450), (128, 300, 130), (64, 130, 1)])
+def test_threshold_sweep_restricted_to_block_lists(dev, D, S, kv_len):
+    """The sweep over the listed key blocks only.  With every block listed it is the full sweep bit
+    for bit (votes, and both bit forms); with the lists that the threshold of the block maxima
+    gives, the mask differs from the full sweep at most where a block's best score lies within
+    rounding of its row's threshold; a block left out of a list is zero in the output; garbage in
+    the buffers beforehand does not show."""
+    print("case sparse sweep", D, S, kv_len, flush=True)
+    B, H = 1, 3
+    q, k, v = wl.clustered_qkv(B, H, S, D, seed=91, sigma=0.7)
+    qd, kd = to_dev(dev, q, k)
+    kv = kv_len or S
+    Sp = orc.padded_len(S)
+    SB, nb, nkb, n64 = Sp // 128, Sp // 64, orc.ceil_div(kv, 64), orc.ceil_div(S, 64)
+    mx = torch.empty((B, H, 1, Sp), device=dev)
+    dn = torch.empty((B, H, 1, Sp), device=dev)
+    bmx = torch.full((B, H, nb, Sp), float("nan"), device=dev)
+    capi.maxq_denom_blockmax(mx, dn, bmx, qd, kd, kv_len=kv_len)
+    _, pmax = orc.booleanmask_rows(f32(mx), f32(dn), f32(q), f32(k), 1.0, qblk=128, kv_len=kv)
+    pblk = np.stack([pmax[..., 64 * J: min(64 * J + 64, kv)].max(axis=-1) for J in range(nkb)], axis=-1)
+    thr = float(np.quantile(pblk, 0.6)) if nkb > 2 else 0.5 * float(pblk.min())   # about 40 % of the blocks pass
+    full = torch.full((B, H, SB, Sp), -7, dtype=torch.int32, device=dev)
+    capi.booleanmask_128(full, mx, dn, qd, kd, thr, kv_len=kv_len)
+    # every block listed: the same kernel walk in list order
+    allb = torch.arange(nb, dtype=torch.int32, device=dev).expand(B, H, SB, nb).contiguous()
+    alln = torch.full((B, H, SB), nb, dtype=torch.int32, device=dev)
+    got = torch.full_like(full, 55)
+    capi.booleanmask_128_blocks(got, mx, dn, qd, kd, thr, allb, alln, kv_len=kv_len)
+    assert torch.equal(got, full)
+    for qblk, rows in ((128, SB), (64, n64)):
+        pf = torch.full((B, H, rows, Sp // 8), 0xA5, dtype=torch.uint8, device=dev)
+        pg = torch.full((B, H, rows, Sp // 8), 0x5A, dtype=torch.uint8, device=dev)
+        capi.booleanmask_packed(pf, mx, dn, qd, kd, thr, qblk=qblk, kv_len=kv_len)
+        capi.booleanmask_packed_blocks(pg, mx, dn, qd, kd, thr, allb, alln, qblk=qblk, kv_len=kv_len)
+        assert torch.equal(pf, pg)
+    # the lists of the block maxima: same mask, except in blocks whose best key is within rounding of the threshold
+    bi = torch.full((B, H, SB, nb), -1, dtype=torch.int32, device=dev)
+    bc = torch.zeros((B, H, SB), dtype=torch.int32, device=dev)
+    bm = torch.zeros((B, H, SB, nb), dtype=torch.uint8, device=dev)
+    capi.blockmax_to_blocklists(bi, bc, bmx, mx, dn, thr, S, D, qblk=128, blockmask=bm, kv_len=kv_len)
+    got = torch.full_like(full, 55)
+    capi.booleanmask_128_blocks(got, mx, dn, qd, kd, thr, bi, bc, kv_len=kv_len)
+    fm, gm, kept = full.cpu().numpy(), got.cpu().numpy(), bm.cpu().numpy().astype(bool)
+    kept_keys = np.repeat(kept, 64, axis=-1)
+    assert np.array_equal(gm[kept_keys], fm[kept_keys]), "votes of the listed blocks"
+    assert not gm[~kept_keys].any(), "everything else is zero"
+    _, margin = orc.block_mask_from_blockmax(np.nan_to_num(bmx.cpu().numpy(), nan=-np.inf), f32(mx), f32(dn), thr, S, D,
+                                             qblk=128, kv_len=kv)
+    clear = np.repeat(np.abs(margin) > 1e-4, 64, axis=-1)
+    assert np.array_equal(gm[clear], fm[clear])
+    assert (gm != fm).mean() < 1e-4
+    if nkb > 2:
+        assert 0.05 < kept[..., :nkb].mean() < 0.95 and fm.any()
+    # a shorter list (first half of each) zeroes the blocks that were dropped
+    half = torch.clamp(bc // 2, min=0)
+    got2 = torch.full_like(full, 55)
+    capi.booleanmask_128_blocks(got2, mx, dn, qd, kd, thr, bi, half, kv_len=kv_len)
+    g2 = got2.cpu().numpy()
+    bih, hh = bi.cpu().numpy(), half.cpu().numpy()
+    for h in range(H):
+        for i in range(SB):
+            want = np.zeros(Sp, np.int32)
+            for J in bih[0, h, i, : hh[0, h, i]]:
+                want[64 * J: 64 * J + 64] = fm[0, h, i, 64 * J: 64 * J + 64]
+            assert np.array_equal(g2[0, h, i], want), (h, i)
+    # ids outside the row and counts beyond max_blocks are tolerated
+    bad = bi.clone()
+    bad[..., 0] = 10 ** 6
+    got3 = torch.full_like(full, 55)
+    capi.booleanmask_128_blocks(got3, mx, dn, qd, kd, thr, bad, bc + 1000, kv_len=kv_len)
+    assert int(got3.min()) >= 0 and int(got3.max()) <= 8
+
+
 def test_all_index_mask(dev):
     print("case all_index_mask", flush=True)
     B, H, SB, S, ms = 2, 3, 5, 600, 640
