@@ -353,6 +353,65 @@ void booleanmask_128(torch::Tensor booleanmask, torch::Tensor o_max_q, torch::Te
 
 // The threshold sweep with a bit-packed result: packed uint8 [B,H,ceil(S/qblk),mask_stride/8],
 // one bit per (q-block of qblk rows, key), least significant bit first.
+// The sweeps restricted to the 64-key blocks listed per 128-row q-block (blk_idx int32
+// [B,H,ceil(S/128),max_blocks], blk_cnt with B*H*ceil(S/128) entries): everything else is zeroed.
+void check_lists128(const torch::Tensor& blk_idx, const torch::Tensor& blk_cnt, const torch::Tensor& q) {
+  check_aux(blk_idx, "blk_idx", at::kInt, q);
+  check_aux(blk_cnt, "blk_cnt", at::kInt, q);
+  const int64_t SB = (q.size(2) + 127) / 128;
+  TORCH_CHECK(blk_idx.dim() == 4 && blk_idx.size(0) == q.size(0) && blk_idx.size(1) == q.size(1) && blk_idx.size(2) == SB &&
+                  blk_idx.size(3) > 0,
+              "blk_idx must be [B,H,ceil(S/128),max_blocks]");
+  TORCH_CHECK(blk_cnt.numel() == q.size(0) * q.size(1) * SB, "blk_cnt must have B*H*ceil(S/128) entries");
+}
+
+void booleanmask_128_blocks(torch::Tensor booleanmask, torch::Tensor o_max_q, torch::Tensor o_denom, torch::Tensor q,
+                            torch::Tensor k, torch::Tensor blk_idx, torch::Tensor blk_cnt, double threshold, double scale,
+                            int64_t kv_len) {
+  check_bhsd(q, "q", q);
+  check_bhsd(k, "k", q);
+  check_aux(booleanmask, "booleanmask", at::kInt, q);
+  check_aux(o_max_q, "o_max_q", at::kFloat, q);
+  check_aux(o_denom, "o_denom", at::kFloat, q);
+  check_lists128(blk_idx, blk_cnt, q);
+  TORCH_CHECK(booleanmask.dim() == 4 && booleanmask.size(0) == q.size(0) && booleanmask.size(1) == q.size(1) &&
+                  booleanmask.size(2) == (q.size(2) + 127) / 128,
+              "booleanmask must be [B,H,ceil(S/128),mask_stride]");
+  const int64_t need = q.size(0) * q.size(1) * padded128(q.size(2));
+  TORCH_CHECK(o_max_q.numel() == need && o_denom.numel() == need, "o_max_q / o_denom must be [B,H,1,128*ceil(S/128)]");
+  const DeviceGuard guard(q.device());
+  check_status(spattn_booleanmask_128_blocks(booleanmask.data_ptr<int>(), (float)threshold, (int)booleanmask.size(3),
+                                             o_max_q.data_ptr<float>(), o_denom.data_ptr<float>(), q.data_ptr(), k.data_ptr(),
+                                             blk_idx.data_ptr<int>(), blk_cnt.data_ptr<int>(), (int)blk_idx.size(3),
+                                             (int)q.size(0), (int)q.size(1), (int)q.size(2), (int)q.size(3),
+                                             checked_kv_len(kv_len, q), (float)scale, cur_stream()),
+               "booleanmask_128_blocks");
+}
+
+void booleanmask_packed_blocks(torch::Tensor packed, torch::Tensor o_max_q, torch::Tensor o_denom, torch::Tensor q,
+                               torch::Tensor k, torch::Tensor blk_idx, torch::Tensor blk_cnt, double threshold, int64_t qblk,
+                               double scale, int64_t kv_len) {
+  check_bhsd(q, "q", q);
+  check_bhsd(k, "k", q);
+  check_aux(packed, "packed", at::kByte, q);
+  check_aux(o_max_q, "o_max_q", at::kFloat, q);
+  check_aux(o_denom, "o_denom", at::kFloat, q);
+  check_lists128(blk_idx, blk_cnt, q);
+  TORCH_CHECK(qblk == 64 || qblk == 128, "qblk must be 64 or 128");
+  TORCH_CHECK(packed.dim() == 4 && packed.size(0) == q.size(0) && packed.size(1) == q.size(1) &&
+                  packed.size(2) == (q.size(2) + qblk - 1) / qblk,
+              "packed must be [B,H,ceil(S/qblk),mask_stride/8]");
+  const int64_t need = q.size(0) * q.size(1) * padded128(q.size(2));
+  TORCH_CHECK(o_max_q.numel() == need && o_denom.numel() == need, "o_max_q / o_denom must be [B,H,1,128*ceil(S/128)]");
+  const DeviceGuard guard(q.device());
+  check_status(spattn_booleanmask_packed_blocks(packed.data_ptr(), (float)threshold, (int)packed.size(3) * 8, (int)qblk,
+                                                o_max_q.data_ptr<float>(), o_denom.data_ptr<float>(), q.data_ptr(), k.data_ptr(),
+                                                blk_idx.data_ptr<int>(), blk_cnt.data_ptr<int>(), (int)blk_idx.size(3),
+                                                (int)q.size(0), (int)q.size(1), (int)q.size(2), (int)q.size(3),
+                                                checked_kv_len(kv_len, q), (float)scale, cur_stream()),
+               "booleanmask_packed_blocks");
+}
+
 void booleanmask_packed(torch::Tensor packed, torch::Tensor o_max_q, torch::Tensor o_denom, torch::Tensor q,
                         torch::Tensor k, double threshold, int64_t qblk, double scale, int64_t kv_len) {
   check_bhsd(q, "q", q);
@@ -521,6 +580,10 @@ void noop_mask_ex(torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, to
 void noop_mask_packed(torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, double, int64_t, double,
                       int64_t) {}
 void noop_blocklists(torch::Tensor, torch::Tensor, OptTensor, torch::Tensor, int64_t) {}
+void noop_mask_blocks(torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, double,
+                      double, int64_t) {}
+void noop_mask_packed_blocks(torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+                             double, int64_t, double, int64_t) {}
 void noop_fmd_bm(torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, double,
                  int64_t) {}
 void noop_md_bm(torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, double, int64_t) {}
@@ -549,6 +612,8 @@ TORCH_LIBRARY_FRAGMENT(cuda_attn, m) {
   m.def("packedmask_to_blocklists(Tensor(a!) blk_idx, Tensor(b!) blk_cnt, Tensor(c!)? blockmask, Tensor packed, int seq) -> ()");
   m.def("booleanmask_to_blocklists(Tensor(a!) blk_idx, Tensor(b!) blk_cnt, Tensor(c!)? blockmask, Tensor booleanmask, int seq) -> ()");
   m.def("qblock_order(Tensor(a!) order, Tensor counts) -> ()");
+  m.def("booleanmask_128_blocks(Tensor(a!) booleanmask, Tensor o_max_q, Tensor o_denom, Tensor q, Tensor k, Tensor blk_idx, Tensor blk_cnt, float threshold, float scale, int kv_len) -> ()");
+  m.def("booleanmask_packed_blocks(Tensor(a!) packed, Tensor o_max_q, Tensor o_denom, Tensor q, Tensor k, Tensor blk_idx, Tensor blk_cnt, float threshold, int qblk, float scale, int kv_len) -> ()");
   m.def("fullattn_maxq_denom_blockmax(Tensor(a!) o, Tensor(b!) o_max_q, Tensor(c!) o_denom, Tensor(d!) blockmax, Tensor q, Tensor k, Tensor v, float scale, int kv_len) -> ()");
   m.def("maxq_denom_blockmax(Tensor(a!) o_max_q, Tensor(b!) o_denom, Tensor(c!) blockmax, Tensor q, Tensor k, float scale, int kv_len) -> ()");
   m.def("blockmax_to_blocklists(Tensor(a!) blk_idx, Tensor(b!) blk_cnt, Tensor(c!)? blockmask, Tensor blockmax, Tensor o_max_q, Tensor o_denom, float threshold, int seq, int head_dim, int qblk, float scale, int kv_len) -> ()");
@@ -575,6 +640,8 @@ TORCH_LIBRARY_IMPL(cuda_attn, Meta, m) {
   m.impl("packedmask_to_blocklists", noop_blocklists);
   m.impl("booleanmask_to_blocklists", noop_blocklists);
   m.impl("qblock_order", noop2);
+  m.impl("booleanmask_128_blocks", noop_mask_blocks);
+  m.impl("booleanmask_packed_blocks", noop_mask_packed_blocks);
   m.impl("fullattn_maxq_denom_blockmax", noop_fmd_bm);
   m.impl("maxq_denom_blockmax", noop_md_bm);
   m.impl("blockmax_to_blocklists", noop_bm_lists);
@@ -602,6 +669,8 @@ TORCH_LIBRARY_IMPL(cuda_attn, CUDA, m) {
   m.impl("packedmask_to_blocklists", packedmask_to_blocklists);
   m.impl("booleanmask_to_blocklists", booleanmask_to_blocklists);
   m.impl("qblock_order", qblock_order);
+  m.impl("booleanmask_128_blocks", booleanmask_128_blocks);
+  m.impl("booleanmask_packed_blocks", booleanmask_packed_blocks);
   m.impl("fullattn_maxq_denom_blockmax", fullattn_maxq_denom_blockmax);
   m.impl("maxq_denom_blockmax", maxq_denom_blockmax);
   m.impl("blockmax_to_blocklists", blockmax_to_blocklists);
@@ -628,6 +697,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("packedmask_to_blocklists", &packedmask_to_blocklists, "bit-packed mask -> KV-block lists");
   m.def("booleanmask_to_blocklists", &booleanmask_to_blocklists, "vote mask -> KV-block lists");
   m.def("qblock_order", &qblock_order, "work order, longest list first");
+  m.def("booleanmask_128_blocks", &booleanmask_128_blocks, "threshold sweep over listed key blocks, int32 votes");
+  m.def("booleanmask_packed_blocks", &booleanmask_packed_blocks, "threshold sweep over listed key blocks, bit-packed");
   m.def("fullattn_maxq_denom_blockmax", &fullattn_maxq_denom_blockmax, "fullattn_maxq_denom + per-block row maxima");
   m.def("maxq_denom_blockmax", &maxq_denom_blockmax, "maxq_denom + per-block row maxima");
   m.def("blockmax_to_blocklists", &blockmax_to_blocklists, "block maxima -> KV-block lists");

@@ -402,6 +402,34 @@ def qk_blocklists_onepass_cuda(q, k, thresh, qblk=128, kv_len=0):
     return blockmax_to_blocklists_cuda(blockmax, max_q, denom, thresh, q.shape[2], q.shape[3], qblk, kv_len)
 
 
+def qk_bitmask_from_blockmax_cuda(blockmax, max_q, denom, q, k, thresh, blocksz=128, kv_len=0):
+    """The vote mask of qk_bitmask_from_maxq_denom_cuda from the block maxima of the statistics sweep:
+    their threshold gives the key blocks in which a key can pass, and the sweep then multiplies those
+    blocks only (the rest of the mask is zero) - the same votes for a fraction of the work."""
+    B, H, S, D = q.shape
+    blk_idx, blk_cnt = blockmax_to_blocklists_cuda(blockmax, max_q, denom, thresh, S, D, 128, kv_len)
+    mask = torch.empty((B, H, (S + blocksz - 1) // blocksz, max_q.shape[3]), dtype=torch.int32, device=q.device)
+    spattn_interface.booleanmask_128_blocks(mask, max_q.contiguous(), denom.contiguous(), q.contiguous(), k.contiguous(),
+                                            blk_idx, blk_cnt, thresh, 0.0, kv_len)
+    return mask
+
+
+def qk_indexmask_from_blockmax_cuda(blockmax, max_q, denom, q, k, thresh, blocksz=128, kv_len=0):
+    """Key lists (the reference's form) from the block maxima: blocks that can hold a key, the sweep over
+    those blocks, the compaction."""
+    mask = qk_bitmask_from_blockmax_cuda(blockmax, max_q, denom, q, k, thresh, blocksz, kv_len)
+    return bitmask_to_indexmask_cuda(mask, kv_len or q.shape[2])
+
+
+def qk_indexmask_onepass_cuda(q, k, thresh, blocksz=128, kv_len=0):
+    """qk_indexmask_cuda with one full sweep over Q K^T instead of two (statistics with block maxima,
+    then the threshold sweep over the blocks that can hold a key)."""
+    max_q, denom = _stats_buffers(q)
+    blockmax = blockmax_buffer(q)
+    spattn_interface.maxq_denom_blockmax(max_q, denom, blockmax, q.contiguous(), k.contiguous(), 0.0, kv_len)
+    return qk_indexmask_from_blockmax_cuda(blockmax, max_q, denom, q, k, thresh, blocksz, kv_len)
+
+
 def qk_blocklists(q, k, thresh=0.001, qblk=128):
     """Pure-torch definition of the block lists: block J of q-block I is kept when some row of I
     and some key of J have softmax > thresh.  Returns (blk_idx padded with -1, blk_cnt, blockmask)."""

@@ -102,12 +102,23 @@ def sparse_attn_from_cache_cuda(query, key, value, *args, **kwargs):
 
 def cached_attn_cuda(query, key, value, current_layer, ditrun, *args, **kwargs):
     """On the steps that refresh the cache: dense attention with statistics, then the mask
-    pre-pass; on every other step: sparse attention from the cached lists (:95-114)."""
+    pre-pass; on every other step: sparse attention from the cached lists (:95-114).
+    ``onepass=True`` (not in the reference): the refresh step sweeps Q K^T once in full instead of twice."""
     mask_cache = kwargs["mask_cache"]
     if mask_cache.run_fullattn(ditrun):
-        out, max_q, denom = _dense_with_stats(query, key, value)
-        kv_indices, kv_num_indices = mask_utils.qk_indexmask_from_maxq_denom_cuda(
-            max_q, denom, query, key, kwargs["thresh"], blocksz=kwargs["blocksz"])
+        if kwargs.get("onepass", False):
+            # the dense pass also writes the block maxima; the threshold sweep then runs over the key
+            # blocks that can hold a key only (same votes, same lists)
+            out = _out_like(query)
+            max_q, denom = mask_utils._stats_buffers(query)
+            blockmax = mask_utils.blockmax_buffer(query)
+            spattn_interface.fullattn_maxq_denom_blockmax(out, max_q, denom, blockmax, *_c(query, key, value), 0.0, 0)
+            kv_indices, kv_num_indices = mask_utils.qk_indexmask_from_blockmax_cuda(
+                blockmax, max_q, denom, query, key, kwargs["thresh"], blocksz=kwargs["blocksz"])
+        else:
+            out, max_q, denom = _dense_with_stats(query, key, value)
+            kv_indices, kv_num_indices = mask_utils.qk_indexmask_from_maxq_denom_cuda(
+                max_q, denom, query, key, kwargs["thresh"], blocksz=kwargs["blocksz"])
         mask_cache.update_cache(current_layer, kv_indices, kv_num_indices)
         return out
     kv_indices, kv_num_indices = mask_cache.get_mask_from_cache(current_layer)

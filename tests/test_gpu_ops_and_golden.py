@@ -267,6 +267,21 @@ def test_block_maxima_operators_and_helpers(dev):
         band = np.abs(pblk - thr) <= 1e-2 * thr
         assert np.array_equal(bm.cpu().numpy().astype(bool) | band, bm_two.cpu().numpy().astype(bool) | band)
         assert 0.05 < bm.float().mean().item() < 0.95
+    # key lists with one full sweep: the reference's form of the lists, equal to the two-sweep lists
+    # except where a block's best key lies within rounding of the threshold
+    i1, n1 = mu.qk_indexmask_onepass_cuda(q, k, thr)
+    i2, n2 = mu.qk_indexmask_cuda(q, k, thr)
+    assert (n1 != n2).float().mean().item() < 0.02 and (i1 != i2).float().mean().item() < 1e-3
+    m1 = mu.qk_bitmask_from_blockmax_cuda(bmx, mx, dn, q, k, thr)
+    m2 = mu.qk_bitmask_from_maxq_denom_cuda(mx, dn, q, k, thr)
+    assert (m1 != m2).float().mean().item() < 1e-4 and int(m1.max()) <= 8 and bool((m1 > 0).any())
+    pk1 = torch.empty((B, H, orc.ceil_div(S, 64), Sp // 8), dtype=torch.uint8, device=dev)
+    b128, c128 = mu.blockmax_to_blocklists_cuda(bmx, mx, dn, thr, S, D, 128)
+    ops.booleanmask_packed_blocks(pk1, mx, dn, q, k, b128, c128, thr, 64, 0.0, 0)
+    pk2 = mu.qk_packedmask_from_maxq_denom_cuda(mx, dn, q, k, thr, 64)
+    assert (pk1 != pk2).float().mean().item() < 1e-3
+    with pytest.raises(RuntimeError):
+        ops.booleanmask_128_blocks(m1, mx, dn, q, k, b128[:, :, :2].contiguous(), c128, thr, 0.0, 0)
     with pytest.raises(RuntimeError):
         ops.blockmax_to_blocklists(bi, bc, None, bmx[:, :, :3].contiguous(), mx, dn, thr, S, D, 128, 0.0, 0)
     with pytest.raises(RuntimeError):
@@ -284,10 +299,13 @@ def test_functionals_with_mask_cache(dev):
     assert_close_o(f32(fn.baseline_attn_maxq_denom(q, k, v, 0, 0)), f32(dense), "baseline_attn_maxq_denom")
     with pytest.raises(NotImplementedError):
         fn.attn_lshmask_cuda(q, k, v, 0, 0, thresh=0.01, blocksz=128)
+    seen_naive = False
     for cache in (mu.NaiveMaskCache([0]), mu.CompressMaskCache([0]), mu.OffloadMaskCache([0]), mu.BitMaskCache([0]),
-                  mu.CompressedBitMaskCache([0])):
+                  mu.CompressedBitMaskCache([0]), mu.NaiveMaskCache([0])):
         f = fn.cached_attn_cuda if isinstance(cache, mu.NaiveMaskCache) else fn.bitmaskcached_attn_cuda
-        o0 = f(q, k, v, 7, 0, thresh=0.01, blocksz=128, mask_cache=cache)       # step 0: dense + cache fill
+        extra = {"onepass": True} if type(cache) is mu.NaiveMaskCache and seen_naive else {}
+        seen_naive = seen_naive or type(cache) is mu.NaiveMaskCache
+        o0 = f(q, k, v, 7, 0, thresh=0.01, blocksz=128, mask_cache=cache, **extra)   # step 0: dense + cache fill
         assert_close_o(f32(o0), f32(dense), "cache fill step")
         o1 = f(q, k, v, 7, 1, thresh=0.01, blocksz=128, mask_cache=cache)       # step 1: sparse from cache
         kvi, kvn = cache.get_mask_from_cache(7)
