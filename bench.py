@@ -318,6 +318,9 @@ def bench_cfg4_end_to_end(dev, steps, warmup, seed=0):
       blockmax128 / blockmax64  one sweep: the statistics pass also writes per-(row, key block) score maxima,
                 whose threshold gives the block lists (prepass_plus_attention_ms counts what the extra output
                 costs the statistics sweep instead of a second sweep)
+      tokens_onepass  the reference's key lists from one full sweep: block lists from the maxima, the threshold
+                sweep over the kept blocks only (same votes), compaction, sp_attn
+      tokens_onepass_bits  the same with bit-packed votes and the key lists decoded from the bits
     Every attention launch uses the work order computed (untimed here, timed on its own) from its counts."""
     c = wl.CONFIGS["cfg4_threshold_padded"]
     B, H, S, D = c["B"], c["H"], c["S"], c["D"]
@@ -436,6 +439,42 @@ def bench_cfg4_end_to_end(dev, steps, warmup, seed=0):
             "sp_attn_blocks_mfma_frac": fl / ms_at / 1e9 / PEAK_BF16_TFLOPS,
             "extra_sweep_ms": ms_mb - out["maxq_denom"]["ms"],
             "prepass_plus_attention_ms": (ms_mb - out["maxq_denom"]["ms"]) + ms_bl + ms_order + ms_at}
+    # route 6: the reference's key lists with one full sweep - block lists (128-row q-blocks) from the maxima,
+    # then the threshold sweep over the kept blocks only, then the compaction as in route 1
+    bi8 = torch.full((B, H, SB, nb), -1, dtype=torch.int32, device=dev)
+    bc8 = torch.zeros((B, H, SB), dtype=torch.int32, device=dev)
+    capi.blockmax_to_blocklists(bi8, bc8, bmx, mx, dn, tau, S, D, qblk=128)
+    del bmx
+    mask = torch.empty((B, H, SB, Sp), dtype=torch.int32, device=dev)
+    ms_sp, _ = time_steps(lambda: capi.booleanmask_128_blocks(mask, mx, dn, q, k, tau, bi8, bc8), steps, warmup)
+    cp = bench_compaction(dev, steps, warmup, mask=mask)
+    kvn2 = torch.zeros((B, H, SB), dtype=torch.int32, device=dev)
+    kvi = torch.full((B, H, SB, Sp), Sp, dtype=torch.int32, device=dev)
+    capi.booleanmask_to_indexmask(kvi, kvn2, mask, S)
+    kept_blocks = int(bc8.sum().item())
+    sp_flops = 2.0 * kept_blocks * 128 * 64 * D
+    out["tokens_onepass"] = {
+        "blockmax_to_blocklists_ms": out["blockmax128"]["blockmax_to_blocklists_ms"],
+        "booleanmask_128_blocks_ms": ms_sp, "booleanmask_128_blocks_tflops": sp_flops / ms_sp / 1e9,
+        "booleanmask_128_blocks_write_gbps": 4.0 * mask.numel() / ms_sp / 1e6,
+        "booleanmask_to_indexmask_ms": cp["ms"], "kept_keys": int(kvn2.sum().item()),
+        "same_counts_as_two_sweeps": bool(torch.equal(kvn2, kvn)),
+        "extra_sweep_ms": ms_mb - out["maxq_denom"]["ms"],
+        "prepass_plus_attention_ms": (ms_mb - out["maxq_denom"]["ms"]) + out["blockmax128"]["blockmax_to_blocklists_ms"]
+                                     + ms_sp + cp["ms"] + ms_order + ms_attn}
+    # route 7: the same with the votes as bits (1/32 of the bytes) and the key lists decoded from the bits
+    del mask
+    pk8 = torch.empty((B, H, SB, Sp // 8), dtype=torch.uint8, device=dev)
+    ms_pb, _ = time_steps(lambda: capi.booleanmask_packed_blocks(pk8, mx, dn, q, k, tau, bi8, bc8, qblk=128), steps, warmup)
+    kvn3 = torch.zeros((B, H, SB), dtype=torch.int32, device=dev)
+    ms_dec, _ = time_steps(lambda: capi.packedmask_to_indexmask(kvi, kvn3, pk8, S), steps, warmup)
+    out["tokens_onepass_bits"] = {
+        "blockmax_to_blocklists_ms": out["blockmax128"]["blockmax_to_blocklists_ms"],
+        "booleanmask_packed_blocks_ms": ms_pb, "booleanmask_packed_blocks_tflops": sp_flops / ms_pb / 1e9,
+        "packedmask_to_indexmask_ms": ms_dec, "same_counts_as_two_sweeps": bool(torch.equal(kvn3, kvn)),
+        "extra_sweep_ms": ms_mb - out["maxq_denom"]["ms"],
+        "prepass_plus_attention_ms": (ms_mb - out["maxq_denom"]["ms"]) + out["blockmax128"]["blockmax_to_blocklists_ms"]
+                                     + ms_pb + ms_dec + ms_order + ms_attn}
     assert torch.isfinite(o.float()).all().item(), "non-finite attention output"
     return out
 

@@ -418,6 +418,37 @@ def test_cfg4_block_maxima_route(dev):
                 continue
             pp, den, _ = orc._softmax_rows(f32(q[0, h, r]) @ kf[0, h, lst].T, 0.125, True)
             assert_close_o(f32(o[0, h, r]), (pp @ vf[0, h, lst]) / den[:, None], "cfg4 blockmax route q%d (%d,%d)" % (qblk, h, j))
+    # the threshold sweep over the listed blocks only gives the votes of the full sweep, bit for bit,
+    # as int32 and as bits, and the key lists of both are the same
+    print("case cfg4 block-restricted threshold sweep", flush=True)
+    del bmx, o
+    SB = Sp // 128
+    bi, bc, _ = lists[128]
+    full = torch.full((B, H, SB, Sp), 7, dtype=torch.int32, device=dev)
+    part = torch.full((B, H, SB, Sp), 7, dtype=torch.int32, device=dev)
+    capi.booleanmask_128(full, mx, dn, qd, kd, thr)
+    capi.booleanmask_128_blocks(part, mx, dn, qd, kd, thr, bi, bc)
+    assert torch.equal(full, part)
+    assert 0 < int(full.count_nonzero()) < full.numel() // 50
+    for qblk in (128, 64):
+        nq = orc.ceil_div(S, qblk)
+        pf = torch.full((B, H, nq, Sp // 8), 0xA5, dtype=torch.uint8, device=dev)
+        pp_ = torch.full((B, H, nq, Sp // 8), 0xA5, dtype=torch.uint8, device=dev)
+        capi.booleanmask_packed(pf, mx, dn, qd, kd, thr, qblk=qblk)
+        capi.booleanmask_packed_blocks(pp_, mx, dn, qd, kd, thr, bi, bc, qblk=qblk)
+        assert torch.equal(pf, pp_), "packed votes, q-blocks of %d" % qblk
+    kvi_f = torch.full((B, H, SB, Sp), -5, dtype=torch.int32, device=dev)
+    kvi_p = torch.full((B, H, SB, Sp), -5, dtype=torch.int32, device=dev)
+    kvn_f, kvn_p = (torch.full((B, H, SB), -5, dtype=torch.int32, device=dev) for _ in range(2))
+    capi.booleanmask_to_indexmask(kvi_f, kvn_f, full, S)
+    del full
+    pk = torch.empty((B, H, SB, Sp // 8), dtype=torch.uint8, device=dev)
+    capi.booleanmask_packed_blocks(pk, mx, dn, qd, kd, thr, bi, bc, qblk=128)
+    capi.packedmask_to_indexmask(kvi_p, kvn_p, pk, S)
+    assert torch.equal(kvn_f, kvn_p)
+    ar = torch.arange(Sp, device=dev, dtype=torch.int32)
+    live = ar[None, None, None, :] < kvn_f[..., None]
+    assert torch.equal(torch.where(live, kvi_f, 0), torch.where(live, kvi_p, 0))
 
 
 def test_reference_shape_75856_with_its_kv_length(dev):
