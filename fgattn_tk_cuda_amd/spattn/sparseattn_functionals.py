@@ -103,10 +103,12 @@ def sparse_attn_from_cache_cuda(query, key, value, *args, **kwargs):
 def cached_attn_cuda(query, key, value, current_layer, ditrun, *args, **kwargs):
     """On the steps that refresh the cache: dense attention with statistics, then the mask
     pre-pass; on every other step: sparse attention from the cached lists (:95-114).
-    ``onepass=True`` (not in the reference): the refresh step sweeps Q K^T once in full instead of twice."""
+    The refresh step sweeps Q K^T once in full instead of twice (the dense pass also writes the score
+    maximum of every row over every 64-key block, S*S/16 bytes per head, freed on return); the lists
+    are the same.  ``onepass=False`` runs the reference's sequence of two full sweeps."""
     mask_cache = kwargs["mask_cache"]
     if mask_cache.run_fullattn(ditrun):
-        if kwargs.get("onepass", False):
+        if kwargs.get("onepass", True):
             # the dense pass also writes the block maxima; the threshold sweep then runs over the key
             # blocks that can hold a key only (same votes, same lists)
             out = _out_like(query)
