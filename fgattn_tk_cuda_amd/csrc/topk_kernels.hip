@@ -8,7 +8,7 @@
 // threshold pre-pass:
 //   qblock_mean_kernel   q -> qmean [B,H,SB,D] bf16 (fp32 sum, * 1/rows, bf16, / sqrt(D), bf16)
 //   qmean_scores_kernel  qmean, k -> score [B,H,SB,score_stride] bf16 (MFMA, fp32 accumulate)
-//   topk_select_kernel   score -> per row the select_k largest, as an ASCENDING key list
+//   topk_select_reg_kernel / topk_select_kernel   score -> per row the select_k largest, as an ASCENDING key list
 // The selection is a two-level radix select on the 16 score bits (two 256-bin histograms)
 // followed by an ordered emit; among equal scores the lower key index wins.  The reference
 // returns the same keys ordered by descending score (ties in whatever order torch.topk
@@ -197,8 +197,9 @@ __device__ __forceinline__ uint32_t order_key(uint32_t bits) {
 
 // The same for the two scores packed in one 32-bit word.
 __device__ __forceinline__ uint32_t order_key2(uint32_t x) {
-  const uint32_t sign = (x >> 15) & 0x00010001u;
-  return x ^ (0x80008000u | (sign * 0x7fffu));
+  typedef short i16x2 __attribute__((ext_vector_type(2)));
+  const i16x2 sign = __builtin_bit_cast(i16x2, x) >> 15;   // 0xffff under a set sign bit
+  return x ^ (0x80008000u | __builtin_bit_cast(uint32_t, sign));
 }
 
 // Exclusive prefix sum over the lanes of per-lane counts below 16, and their total: one
@@ -352,46 +353,139 @@ __global__ __launch_bounds__(256) void topk_select_kernel(int* __restrict__ kv_i
   }
 }
 
-// The same selection with the row held in LDS: one workgroup per row reads its scores from
-// HBM once, keeps them as 16-bit keys (2 bytes per key), and runs the passes out of LDS.  Wave w
-// emits its contiguous part of the row; where its part of the list starts follows from the
-// parts' counts of scores above and equal to the threshold.  Used while the row fits
-// (kv_len <= kTopkLdsMaxKeys); longer rows take topk_select_kernel.
-constexpr int kTopkLdsMaxKeys = 72000;
-// A score row has few distinct exponents: most keys of a pass land in a handful of bins.  Every
-// bin is therefore kept as 4 partial counts, one per lane & 3, next to each other (4
-// different banks): the adds of a wave to one bin meet 16 to an address instead of 64.
-constexpr int kTopkSubs = 4;
-constexpr int kTopkThreads = 512;
-constexpr int kTopkWaves = kTopkThreads / 64;
-constexpr int kTopkLdsExtra = 256 * kTopkSubs * 4 + kTopkWaves * 2 * 4;   // histogram + per-wave counts
+// ------------------------------------------------------------------------------------
+// The same selection with the row held in registers: one workgroup of 512 lanes per row, every
+// lane keeps VPL 16-byte vectors (8 keys each) of the row as packed 16-bit keys from the one HBM
+// read to the emit.  Wave w owns the vectors [64 VPL w, 64 VPL (w + 1)), lane l of it the
+// vectors 64 VPL w + 64 u + l: a wave-wide load is 1 KB contiguous, and (wave, u, lane, element)
+// is the key order.  LDS holds only the histogram: every bin as 32 partial counts, one per
+// lane & 31, next to each other - a wave's adds to one bin go to 32 different banks and meet at
+// most two to an address, however few bins the row's exponents fill.  Two keys are handled per
+// instruction wherever the 16-bit packed forms allow it (key order, pass-2 bin, the
+// above / equal flags of the emit, which one dot product per register turns into a bit mask),
+// and the lane prefix sums of the emit run on counts packed two to a register.
+// ------------------------------------------------------------------------------------
+constexpr int kRegThreads = 512;
+constexpr int kRegSlots = 32;
+constexpr int kRegSlotShift = 5;
+constexpr int kRegMaxVpl = 18;
+constexpr int kRegMaxKeys = kRegThreads * kRegMaxVpl * 8;   // 73728
 
-__global__ __launch_bounds__(kTopkThreads) void topk_select_lds_kernel(int* __restrict__ kv_indices, int* __restrict__ kv_num,
-                                                               const uint16_t* __restrict__ score, int rows,
-                                                               int score_stride, int kv_len, int select_k,
-                                                               int idx_stride) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  const int nvec = (kv_len + 7) >> 3;
-  u32x4* keys = reinterpret_cast<u32x4*>(smem_raw);                       // nvec vectors of 8 keys
-  unsigned* hist = reinterpret_cast<unsigned*>(smem_raw + 16 * (size_t)nvec);
-  int* wave_cnt = reinterpret_cast<int*>(hist + 256 * kTopkSubs);          // [waves][2]: above, equal
-  constexpr int NTHR = kTopkThreads;
+__device__ __forceinline__ uint32_t pk_sub_sat_u16(uint32_t a, uint32_t b) {
+  uint32_t d;
+  asm("v_pk_sub_u16 %0, %1, %2 clamp" : "=v"(d) : "v"(a), "v"(b));
+  return d;
+}
+__device__ __forceinline__ uint32_t pk_sub_u16(uint32_t a, uint32_t b) {
+  uint32_t d;
+  asm("v_pk_sub_u16 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b));
+  return d;
+}
+__device__ __forceinline__ uint32_t pk_min_u16(uint32_t a, uint32_t b) {
+  uint32_t d;
+  asm("v_pk_min_u16 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b));
+  return d;
+}
+__device__ __forceinline__ uint32_t pk_mad_u16(uint32_t a, uint32_t b, uint32_t c) {
+  uint32_t d;
+  asm("v_pk_mad_u16 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+  return d;
+}
+// adds 1 to the 32-bit LDS word at a byte address
+__device__ __forceinline__ void lds_add_one(uint32_t byte_addr) {
+  __hip_atomic_fetch_add((SPATTN_LDS unsigned*)(uintptr_t)byte_addr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+// acc + lo16(flags) * lo16(weights) + hi16(flags) * hi16(weights)
+__device__ __forceinline__ uint32_t dot2_u16(uint32_t flags, uint32_t weights, uint32_t acc) {
+  typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+  return __builtin_amdgcn_udot2(__builtin_bit_cast(u16x2, flags), __builtin_bit_cast(u16x2, weights), acc, false);
+}
+// Inclusive prefix sum over the 64 lanes (fields packed in x must not carry into each other).
+__device__ __forceinline__ uint32_t lane_scan(uint32_t x) {
+  int v = (int)x;
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, true);   // row_shr:1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, true);   // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, true);   // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, true);   // row_shr:8
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1 and 3
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2 and 3
+  return (uint32_t)v;
+}
+
+// find_bin on plain counts with the bins dealt to the lanes from the top (lane l holds bins
+// 255 - 4l .. 252 - 4l): the sum over the bins at and above a lane's own is then an inclusive
+// prefix sum over the lanes, six DPP adds instead of six cross-lane reads through LDS.
+__device__ __forceinline__ void find_bin_top_down(const unsigned* tot, int lane, int need, int& bin, int& above) {
+  const u32x4 c = *reinterpret_cast<const u32x4*>(tot + 252 - 4 * lane);   // c[3] is the highest bin of the four
+  const int own = (int)(c[0] + c[1] + c[2] + c[3]);
+  const int s = (int)lane_scan((uint32_t)own);
+  const unsigned long long m = __ballot(s >= need);           // m != 0 because need <= total
+  const int L = __builtin_ctzll(m);
+  int a = s - own;                                            // strictly above this lane's bins
+  int b = 252 - 4 * lane;
+#pragma unroll
+  for (int i = 3; i >= 0; --i) {
+    if (a + (int)c[i] >= need) { b = 252 - 4 * lane + i; break; }
+    a += (int)c[i];
+  }
+  bin = __builtin_amdgcn_readlane(b, L);
+  above = __builtin_amdgcn_readlane(a, L);
+}
+
+// Sums the 32 partial counts of every bin into tot[256], clears what it read (and the overflow
+// bin when asked), and finds the bin that holds the need-th largest key.  Two barriers inside;
+// the caller has put one behind the last add.
+template <bool CLEAR_OVERFLOW>
+__device__ __forceinline__ void reduce_and_find(unsigned* hist, unsigned* tot, int tid, int lane, int need, int& bin,
+                                                int& above) {
+  u32x4* p = reinterpret_cast<u32x4*>(hist + (tid >> 1) * kRegSlots + (tid & 1) * (kRegSlots / 2));
+  const u32x4 zero = {0, 0, 0, 0};
+  unsigned s = 0;
+  // a lane's 64 bytes start 16 banks from its neighbour's: neighbouring pairs of lanes take their
+  // four 16-byte pieces in rotated order, so that 16 lanes cover all banks in every step
+#pragma unroll
+  for (int j = 0; j < kRegSlots / 8; ++j) {
+    const int jj = (j + (tid >> 1)) & (kRegSlots / 8 - 1);
+    const u32x4 c = p[jj];
+    p[jj] = zero;
+    s += c[0] + c[1] + c[2] + c[3];
+  }
+  s += __shfl_xor(s, 1, 64);
+  if (!(tid & 1)) tot[tid >> 1] = s;
+  if (CLEAR_OVERFLOW && tid < kRegSlots) hist[256 * kRegSlots + tid] = 0;
+  __syncthreads();
+  find_bin_top_down(tot, lane, need, bin, above);
+  __syncthreads();   // tot is rewritten by the next reduction
+}
+
+template <int VPL>
+__global__ __launch_bounds__(kRegThreads) __attribute__((amdgpu_waves_per_eu(VPL <= 8 ? 6 : (VPL <= 12 ? 4 : 2)))) void topk_select_reg_kernel(int* __restrict__ kv_indices, int* __restrict__ kv_num,
+                                                                     const uint16_t* __restrict__ score, int rows,
+                                                                     int score_stride, int kv_len, int select_k,
+                                                                     int idx_stride) {
+  __shared__ __attribute__((aligned(16))) unsigned hist[257 * kRegSlots];   // bin 256: pass-2 keys outside the pass-1 bin
+  __shared__ __attribute__((aligned(16))) unsigned tot[256];
+  __shared__ unsigned wave_cnt[kRegThreads / 64];
+  constexpr int NP = (VPL + 1) / 2;   // registers of counts packed two to a register
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int sub = tid & (kTopkSubs - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nvec = (kv_len + 7) >> 3;
   int want = select_k < kv_len ? select_k : kv_len;
   want = want < idx_stride ? want : idx_stride;
-  // wave w owns vectors [w * per, (w + 1) * per), per a multiple of 64
-  const int per = ((nvec + NTHR - 1) / NTHR) << 6;
-  const int v_lo = wave * per;
-  const int v_hi = (v_lo + per) < nvec ? (v_lo + per) : nvec;
+  const int vbase = wave * (VPL * 64) + lane;
+  // the vector that holds key kv_len - 1, when elements behind kv_len share it: its wave, slot and lane
+  const int tail_wave = (kv_len & 7) ? (nvec - 1) / (VPL * 64) : -1;
+  const int tail_u = ((nvec - 1) % (VPL * 64)) >> 6;
+  const int tail_lane = (nvec - 1) & 63;
+  unsigned* const my_hist = hist + (lane & (kRegSlots - 1));
+  SPATTN_LDS unsigned* const my_hist_lds = (SPATTN_LDS unsigned*)my_hist;
+  const uint32_t one2 = 0x00010001u;
 
-  auto key16 = [](const u32x4& x, int e) -> uint32_t {
-    const uint32_t w = x[e >> 1];
-    return (e & 1) ? (w >> 16) : (w & 0xffffu);
-  };
-
+  {
+    const u32x4 zero = {0, 0, 0, 0};
+    for (int i = tid; i < 257 * kRegSlots / 4; i += kRegThreads) reinterpret_cast<u32x4*>(hist)[i] = zero;
+  }
   for (int row = blockIdx.x; row < rows; row += gridDim.x) {
     const u32x4* __restrict__ src = reinterpret_cast<const u32x4*>(score + (size_t)row * score_stride);
     int* __restrict__ dst = kv_indices + (size_t)row * idx_stride;
@@ -399,126 +493,176 @@ __global__ __launch_bounds__(kTopkThreads) void topk_select_lds_kernel(int* __re
       if (tid == 0) kv_num[row] = 0;
       continue;
     }
-    for (int i = tid; i < 256 * kTopkSubs; i += NTHR) hist[i] = 0;
-    __syncthreads();
-    // Load, convert, pass 1 (high bytes).  Eight loads in flight per lane: the adds keep the
-    // compiler from moving a load across them, and one load per trip would expose the memory
-    // latency on every trip.  The up to 7 elements behind kv_len in the last vector get key
-    // 0, the smallest, and are then treated like keys: with the largest indices of the row
-    // they are the last candidates among equal keys, and want <= kv_len never reaches them.
-    constexpr int U = 8;
-    for (int v0 = tid; v0 < nvec; v0 += NTHR * U) {
-      u32x4 xs[U];
+    // Vectors behind the row hold the bit pattern whose key is 0, the smallest; so do the up to 7
+    // elements behind kv_len in the last vector.  They count as keys: with the largest indices of
+    // the row they are the last candidates among equal keys, and want <= kv_len never reaches them.
+    u32x4 y[VPL];
+    if ((wave + 1) * (VPL * 64) <= nvec) {
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const int v = v0 + NTHR * u;
-        const u32x4 z = {0, 0, 0, 0};
-        xs[u] = v < nvec ? __builtin_nontemporal_load(src + v) : z;
-      }
+      for (int u = 0; u < VPL; ++u) y[u] = __builtin_nontemporal_load(src + vbase + 64 * u);
+    } else {
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const int v = v0 + NTHR * u;
-        if (v < nvec) {
-          u32x4 y;
-#pragma unroll
-          for (int h = 0; h < 4; ++h) y[h] = order_key2(xs[u][h]);
-          if (8 * v + 8 > kv_len) {
-#pragma unroll
-            for (int h = 0; h < 4; ++h) {
-              if (8 * v + 2 * h >= kv_len) y[h] &= 0xffff0000u;
-              if (8 * v + 2 * h + 1 >= kv_len) y[h] &= 0x0000ffffu;
-            }
-          }
-          keys[v] = y;
-#pragma unroll
-          for (int e = 0; e < 8; ++e) atomicAdd(&hist[(key16(y, e) >> 8) * kTopkSubs + sub], 1u);
-        }
+      for (int u = 0; u < VPL; ++u) {
+        const int v = vbase + 64 * u;
+        const u32x4 lowest = {~0u, ~0u, ~0u, ~0u};
+        y[u] = v < nvec ? __builtin_nontemporal_load(src + v) : lowest;
       }
     }
+#pragma unroll
+    for (int u = 0; u < VPL; ++u)
+#pragma unroll
+      for (int h = 0; h < 4; ++h) y[u][h] = order_key2(y[u][h]);
+    if (wave == tail_wave) {
+      const int left = kv_len & 7;   // elements of the vector that are keys
+#pragma unroll
+      for (int u = 0; u < VPL; ++u)
+        if (u == tail_u) {
+#pragma unroll
+          for (int h = 0; h < 4; ++h) {
+            const uint32_t keep = 2 * h + 1 < left ? ~0u : (2 * h < left ? 0x0000ffffu : 0u);
+            y[u][h] &= lane == tail_lane ? keep : ~0u;
+          }
+        }
+    }
+    __syncthreads();   // the histogram is clear
+    // pass 1: high bytes
+#pragma unroll
+    for (int u = 0; u < VPL; ++u)
+#pragma unroll
+      for (int h = 0; h < 4; ++h) {
+        const uint32_t w = y[u][h];
+        atomicAdd(my_hist + ((w >> 24) << kRegSlotShift), 1u);
+        atomicAdd(my_hist + (((w >> 8) & 0xffu) << kRegSlotShift), 1u);
+      }
     __syncthreads();
     int b1, gt1;
-    find_bin<kTopkSubs>(hist, lane, want, b1, gt1);   // every wave finds the same bin
-    __syncthreads();
-    for (int i = tid; i < 256 * kTopkSubs; i += NTHR) hist[i] = 0;
-    __syncthreads();
-    // pass 2 (low bytes under high byte b1)
-    for (int v = tid; v < nvec; v += NTHR) {
-      const u32x4 y = keys[v];
+    reduce_and_find<false>(hist, tot, tid, lane, want, b1, gt1);
+    // pass 2: low bytes under high byte b1; every other key goes to bin 256
+    {
+      const uint32_t base2 = (uint32_t)b1 * 0x01000100u;
+      const uint32_t cap2 = 0x01000100u;
+      const uint32_t stride2 = (4u * kRegSlots) * 0x00010001u;                       // bytes per bin
+      const uint32_t slot2 = (uint32_t)(uintptr_t)my_hist_lds * 0x00010001u;          // this lane's count of bin 0
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const uint32_t key = key16(y, e);
-        if ((int)(key >> 8) == b1) atomicAdd(&hist[(key & 255u) * kTopkSubs + sub], 1u);
-      }
+      for (int u = 0; u < VPL; ++u)
+#pragma unroll
+        for (int h = 0; h < 4; ++h) {
+          // both LDS addresses of the register's two keys in one packed multiply-add (all below 64 KB)
+          const uint32_t a2 = pk_mad_u16(pk_min_u16(pk_sub_u16(y[u][h], base2), cap2), stride2, slot2);
+          lds_add_one(a2 & 0xffffu);
+          lds_add_one(a2 >> 16);
+        }
     }
     __syncthreads();
     int b2, gt2;
-    find_bin<kTopkSubs>(hist, lane, want - gt1, b2, gt2);
+    reduce_and_find<true>(hist, tot, tid, lane, want - gt1, b2, gt2);
     const uint32_t T = ((uint32_t)b1 << 8) | (uint32_t)b2;
-    const int r = want - gt1 - gt2;
-    // counts of this wave's part
-    int cg = 0, ce = 0;
-    for (int v = v_lo + lane; v < v_hi; v += 64) {
-      const u32x4 y = keys[v];
+    const int r = want - gt1 - gt2;   // keys equal to T that are still needed, in key order
+
+    // per vector: bit 2e of gtm / eqm says that element e lies above / at the threshold.  Both come
+    // from one 2-bit field per element, min(key - (T - 1), 2) with the difference saturating at 0:
+    // 0 below T, 1 at T, 2 above; one dot product per register puts its two fields in place.
+    uint32_t gtm[VPL], eqm[VPL];
+    {
+      const uint32_t Tu = (uint32_t)__builtin_amdgcn_readfirstlane((int)T);
+      const uint32_t two2 = 0x00020002u;
+      const uint32_t below2 = (Tu - 1u) * 0x00010001u;
+      if (Tu) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const uint32_t key = key16(y, e);
-        cg += key > T ? 1 : 0;
-        ce += key == T ? 1 : 0;
-      }
-    }
+        for (int u = 0; u < VPL; ++u) {
+          uint32_t f = 0;
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-      cg += __shfl_xor(cg, off, 64);
-      ce += __shfl_xor(ce, off, 64);
-    }
-    if (lane == 0) {
-      wave_cnt[2 * wave] = cg;
-      wave_cnt[2 * wave + 1] = ce;
-    }
-    __syncthreads();
-    int gt_start = 0, eq_seen = 0;
-    for (int u = 0; u < wave; ++u) {
-      gt_start += wave_cnt[2 * u];
-      eq_seen += wave_cnt[2 * u + 1];
-    }
-    int out_pos = gt_start + (eq_seen < r ? eq_seen : r);
-    // ordered emit of this wave's part
-    for (int v0 = v_lo; v0 < v_hi; v0 += 64) {
-      const int v = v0 + lane;
-      unsigned gt = 0, eq = 0;
-      if (v < v_hi) {
-        const u32x4 y = keys[v];
+          for (int h = 0; h < 4; ++h)
+            f = dot2_u16(pk_min_u16(pk_sub_sat_u16(y[u][h], below2), two2), (1u << (4 * h)) | (4u << (4 * h + 16)), f);
+          gtm[u] = (f >> 1) & 0x5555u;
+          eqm[u] = f & 0x5555u;
+        }
+      } else {   // every key is at or above a threshold of 0
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const uint32_t key = key16(y, e);
-          gt |= (key > T ? 1u : 0u) << e;
-          eq |= (key == T ? 1u : 0u) << e;
+        for (int u = 0; u < VPL; ++u) {
+          uint32_t f = 0;
+#pragma unroll
+          for (int h = 0; h < 4; ++h)
+            f = dot2_u16(pk_min_u16(y[u][h], one2) + one2, (1u << (4 * h)) | (4u << (4 * h + 16)), f);
+          gtm[u] = (f >> 1) & 0x5555u;
+          eqm[u] = f & 0x5555u;
         }
       }
-      int eq_before, eq_total;
-      lane_prefix4(__popc(eq), eq_before, eq_total);
-      int keep = r - (eq_seen + eq_before);
-      keep = keep < 0 ? 0 : keep;
-      unsigned eq_kept = 0;
-      while (eq && keep > 0) {
-        eq_kept |= eq & (0u - eq);
-        eq &= eq - 1;
-        --keep;
+    }
+    // where this wave's part of the list starts: counts of the waves before it
+    uint32_t mine = 0;
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) mine += (uint32_t)__popc(gtm[u]) + ((uint32_t)__popc(eqm[u]) << 16);
+    const uint32_t wave_total = (uint32_t)__builtin_amdgcn_readlane((int)lane_scan(mine), 63);
+    if (lane == 0) wave_cnt[wave] = wave_total;
+    __syncthreads();
+    int out_pos = 0, eq_seen = 0;
+    {
+      uint32_t before = 0;
+#pragma unroll
+      for (int u = 0; u < kRegThreads / 64 - 1; ++u) before += u < wave ? wave_cnt[u] : 0u;
+      out_pos = (int)(before & 0xffffu);
+      eq_seen = (int)(before >> 16);
+    }
+    out_pos += eq_seen < r ? eq_seen : r;
+    if (wave_total >> 16) {
+      // keys equal to T in this wave: keep those whose rank among all such keys of the row is below r
+      uint32_t ec[NP];
+#pragma unroll
+      for (int j = 0; j < NP; ++j) {
+        ec[j] = (uint32_t)__popc(eqm[2 * j]);
+        if (2 * j + 1 < VPL) ec[j] += (uint32_t)__popc(eqm[2 * j + 1]) << 16;
+        ec[j] = lane_scan(ec[j]);
       }
-      unsigned sel = gt | eq_kept;
-      int before, total;
-      lane_prefix4(__popc(sel), before, total);
-      int pos = out_pos + before;
+#pragma unroll
+      for (int u = 0; u < VPL; ++u) {
+        const uint32_t incl = (ec[u >> 1] >> (16 * (u & 1))) & 0xffffu;
+        const uint32_t total = ((uint32_t)__builtin_amdgcn_readlane((int)ec[u >> 1], 63) >> (16 * (u & 1))) & 0xffffu;
+        uint32_t e = eqm[u];
+        int keep = r - (eq_seen + (int)incl - __popc(e));
+        uint32_t kept = 0;
+        while (e && keep > 0) {
+          kept |= e & (0u - e);
+          e &= e - 1;
+          --keep;
+        }
+        gtm[u] |= kept;
+        eq_seen += (int)total;
+      }
+    }
+    // ordered emit
+    uint32_t sc[NP];
+#pragma unroll
+    for (int j = 0; j < NP; ++j) {
+      sc[j] = (uint32_t)__popc(gtm[2 * j]);
+      if (2 * j + 1 < VPL) sc[j] += (uint32_t)__popc(gtm[2 * j + 1]) << 16;
+      sc[j] = lane_scan(sc[j]);
+    }
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) {
+      const uint32_t incl = (sc[u >> 1] >> (16 * (u & 1))) & 0xffffu;
+      const uint32_t total = ((uint32_t)__builtin_amdgcn_readlane((int)sc[u >> 1], 63) >> (16 * (u & 1))) & 0xffffu;
+      uint32_t sel = gtm[u];
+      int pos = out_pos + (int)incl - __popc(sel);
+      const int key0 = 8 * (vbase + 64 * u);
       while (sel) {
-        dst[pos++] = 8 * v + __builtin_ctz(sel);
+        dst[pos++] = key0 + (__builtin_ctz(sel) >> 1);
         sel &= sel - 1;
       }
-      out_pos += total;
-      eq_seen += eq_total;
+      out_pos += (int)total;
     }
     if (tid == 0) kv_num[row] = want;
-    __syncthreads();   // the row buffer and the counts are reused
+    // wave_cnt is rewritten only behind the barriers of the next row's passes
   }
+}
+
+template <int VPL>
+static hipError_t launch_topk_select_reg(int* kv_indices, int* kv_num, const uint16_t* score, int rows, int score_stride,
+                                         int kv_len, int select_k, int idx_stride, hipStream_t stream) {
+  const int grid = rows < 16384 ? rows : 16384;
+  hipLaunchKernelGGL(topk_select_reg_kernel<VPL>, dim3(grid), dim3(kRegThreads), 0, stream, kv_indices, kv_num, score, rows,
+                     score_stride, kv_len, select_k, idx_stride);
+  return hipGetLastError();
 }
 
 hipError_t run_topk_mask(int* kv_indices, int* kv_num, uint16_t* score, uint16_t* qmean, const uint16_t* q,
@@ -547,16 +691,17 @@ hipError_t run_topk_mask(int* kv_indices, int* kv_num, uint16_t* score, uint16_t
     e = hipGetLastError();
     if (e != hipSuccess) return e;
   }
-  if (kv_len <= kTopkLdsMaxKeys) {
-    const int lds = 16 * ((kv_len + 7) / 8) + kTopkLdsExtra;
-    static bool attr_set[kMaxDevices] = {};
-    e = raise_lds_limit(reinterpret_cast<const void*>(topk_select_lds_kernel),
-                        16 * (kTopkLdsMaxKeys / 8) + kTopkLdsExtra, attr_set);
-    if (e != hipSuccess) return e;
-    const int grid = rows < 8192 ? rows : 8192;
-    hipLaunchKernelGGL(topk_select_lds_kernel, dim3(grid), dim3(kTopkThreads), lds, stream, kv_indices, kv_num, score, rows,
-                       score_stride, kv_len, select_k, idx_stride);
-    return hipGetLastError();
+  if (kv_len <= kRegMaxKeys) {
+    const int vpl = ((kv_len + 7) / 8 + kRegThreads - 1) / kRegThreads;
+#define SPATTN_TOPK_REG(V) \
+  if (vpl <= V) return launch_topk_select_reg<V>(kv_indices, kv_num, score, rows, score_stride, kv_len, select_k, idx_stride, stream)
+    SPATTN_TOPK_REG(1);
+    SPATTN_TOPK_REG(2);
+    SPATTN_TOPK_REG(4);
+    SPATTN_TOPK_REG(8);
+    SPATTN_TOPK_REG(12);
+    SPATTN_TOPK_REG(18);
+#undef SPATTN_TOPK_REG
   }
   int grid = (rows + 3) / 4;
   if (grid > 4096) grid = 4096;

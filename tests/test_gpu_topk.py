@@ -53,8 +53,40 @@ def test_topk_generator_matches_oracle(dev, D, blk, S, select_k, kv_len):
     assert np.all(kvi[..., kk:] == fill)
 
 
-def test_topk_rows_longer_than_the_lds_path(dev):
-    """More than 72000 keys per row: the select that re-reads its row from memory."""
+@pytest.mark.parametrize("S,select_k", [(4096, 300), (8200, 8100), (16001, 1300), (32757, 2621), (32768, 32768), (45003, 900),
+                                        (72001, 6000), (73728, 73000)])
+def test_topk_select_row_lengths_with_many_ties(dev, S, select_k):
+    """Every row length class of the in-register select (1, 2, 4, 8, 12 and 18 vectors per lane), row
+    ends inside a 16-byte vector, and keys on a coarse grid so that many scores are equal - also at
+    the threshold, where the lower key wins."""
+    print("case topk row lengths", S, select_k, flush=True)
+    B, H, D, blk = 1, 1, 64, 128
+    g = torch.Generator().manual_seed(S)
+    q = (torch.randint(-2, 3, (B, H, S, D), generator=g).float() * 0.5).bfloat16()
+    k = (torch.randint(-2, 3, (B, H, S, D), generator=g).float() * 0.25).bfloat16()
+    kvi, kvn, score, _, fill = _run(dev, q, k, select_k, blk)
+    SB = orc.ceil_div(S, blk)
+    rows = sorted({0, 1, SB // 3, SB // 2, SB - 2, SB - 1})
+    got_sc = score[0, 0, rows, :S]
+    assert np.isfinite(got_sc).all()
+    assert len(np.unique(got_sc[0])) < S // 4          # ties everywhere
+    want_sel = orc.topk_select(got_sc, select_k)
+    kk = min(select_k, S)
+    assert np.all(kvn == kk)
+    assert np.array_equal(kvi[0, 0, rows, :kk], want_sel)
+    assert np.all(kvi[0, 0, :, kk:] == fill)
+    # every row: ascending, in range, and no key left out has a higher score than a key taken
+    lists = kvi[0, 0, :, :kk]
+    assert np.all(np.diff(lists, axis=1) > 0) and lists.min() >= 0 and lists.max() < S
+    for r in range(0, SB, max(1, SB // 16)):
+        taken = np.zeros(S, bool)
+        taken[lists[r]] = True
+        if kk < S:
+            assert score[0, 0, r, :S][taken].min() >= score[0, 0, r, :S][~taken].max()
+
+
+def test_topk_rows_longer_than_the_register_path(dev):
+    """More than 73728 keys per row: the select that re-reads its row from memory."""
     print("case topk long rows", flush=True)
     B, H, S, D, blk, select_k = 1, 1, 81000, 64, 128, 700
     q, k, _ = wl.randn_qkv(B, H, S, D, seed=5)
