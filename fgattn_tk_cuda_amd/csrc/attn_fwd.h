@@ -421,8 +421,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   auto stat_piece = [&](const f32x16 (&s)[NMB], int k, float& mloc) {
     const int mb = k >> 2, r = 4 * (k & 3);
     if (k == 0) mloc = s[0][0];
-    mloc = fmaxf(mloc, fmaxf(s[mb][r], s[mb][r + 1]));
-    mloc = fmaxf(mloc, fmaxf(s[mb][r + 2], s[mb][r + 3]));
+    mloc = max3_raw(mloc, s[mb][r], s[mb][r + 1]);
+    mloc = max3_raw(mloc, s[mb][r + 2], s[mb][r + 3]);
   };
   // tile: the key block the maxima belong to.  With the statistics outputs a caller may also ask
   // for them per key block (blockmax[J][row], raw like max_q): the threshold test of the mask
@@ -433,7 +433,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
     if constexpr (STATS && KSPLIT == 1 && MODE == KV_DENSE) {
       if (p.blockmax != nullptr && g == 0) p.blockmax[((size_t)bh * (p.Sp >> 6) + tile) * p.Sp + qrow] = mloc;
     }
-    m_true = fmaxf(m_true, mloc);
+    m_true = max_raw(m_true, mloc);
     return mloc * p.sf;
   };
   auto row_stats = [&](const f32x16 (&s)[NMB], int tile) -> float {
@@ -445,7 +445,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   // Move the exponent reference if some row of the wave outgrew it; rescales O and l.
   auto maybe_rescale = [&](float mloc_sf) {
     if (__any(mloc_sf > mr_sf + kSlack)) {
-      const float new_sf = fmaxf(mr_sf, mloc_sf);
+      const float new_sf = max_raw(mr_sf, mloc_sf);
       const float alpha = (new_sf == kNegInf) ? 1.f : __builtin_amdgcn_exp2f(mr_sf - new_sf);
       mr_sf = new_sf;
       base_eff = (new_sf == kNegInf) ? kNoRef : new_sf;
