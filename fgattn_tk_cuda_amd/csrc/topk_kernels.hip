@@ -97,7 +97,7 @@ constexpr int kKeysPerWg = 2048;
 constexpr int kScorePitch = 512 + 16;   // bytes per staged row; rows 4 apart land 16 banks apart
 
 template <int D>
-__global__ __launch_bounds__(256) void qmean_scores_kernel(uint16_t* __restrict__ score,
+__global__ __launch_bounds__(256, 2) void qmean_scores_kernel(uint16_t* __restrict__ score,
                                                             const uint16_t* __restrict__ qmean,
                                                             const uint16_t* __restrict__ k, int S, int SB, int kv_len,
                                                             int score_stride) {
