@@ -402,23 +402,45 @@ def qk_blocklists_onepass_cuda(q, k, thresh, qblk=128, kv_len=0):
     return blockmax_to_blocklists_cuda(blockmax, max_q, denom, thresh, q.shape[2], q.shape[3], qblk, kv_len)
 
 
+# The key-list route thresholds the block maxima a little below the vote threshold: the statistics
+# sweep and the vote sweep round a score differently (one rounds s and compares, the other accumulates
+# s - t in the matrix unit), so a key whose margin is within that rounding could otherwise sit in a block
+# the maxima leave out.  tau (1 - 1e-3) moves the block test by about 0.01 raw score units, a hundred times
+# the rounding of either sweep; the few blocks it adds contribute zero votes.
+_BLOCK_THRESH_SLACK = 1.0 - 1e-3
+
+
+def _blocks_that_can_hold_a_key(blockmax, max_q, denom, thresh, S, D, kv_len):
+    return blockmax_to_blocklists_cuda(blockmax, max_q, denom, thresh * _BLOCK_THRESH_SLACK, S, D, 128, kv_len)
+
+
 def qk_bitmask_from_blockmax_cuda(blockmax, max_q, denom, q, k, thresh, blocksz=128, kv_len=0):
     """The vote mask of qk_bitmask_from_maxq_denom_cuda from the block maxima of the statistics sweep:
     their threshold gives the key blocks in which a key can pass, and the sweep then multiplies those
     blocks only (the rest of the mask is zero) - the same votes for a fraction of the work."""
     B, H, S, D = q.shape
-    blk_idx, blk_cnt = blockmax_to_blocklists_cuda(blockmax, max_q, denom, thresh, S, D, 128, kv_len)
+    blk_idx, blk_cnt = _blocks_that_can_hold_a_key(blockmax, max_q, denom, thresh, S, D, kv_len)
     mask = torch.empty((B, H, (S + blocksz - 1) // blocksz, max_q.shape[3]), dtype=torch.int32, device=q.device)
     spattn_interface.booleanmask_128_blocks(mask, max_q.contiguous(), denom.contiguous(), q.contiguous(), k.contiguous(),
                                             blk_idx, blk_cnt, thresh, 0.0, kv_len)
     return mask
 
 
+def qk_packedmask_from_blockmax_cuda(blockmax, max_q, denom, q, k, thresh, qblk=128, kv_len=0):
+    """The same votes as bits (qk_packedmask_from_maxq_denom_cuda over the blocks that can hold a key)."""
+    B, H, S, D = q.shape
+    blk_idx, blk_cnt = _blocks_that_can_hold_a_key(blockmax, max_q, denom, thresh, S, D, kv_len)
+    packed = torch.empty((B, H, (S + qblk - 1) // qblk, max_q.shape[3] // 8), dtype=torch.uint8, device=q.device)
+    spattn_interface.booleanmask_packed_blocks(packed, max_q.contiguous(), denom.contiguous(), q.contiguous(), k.contiguous(),
+                                               blk_idx, blk_cnt, thresh, qblk, 0.0, kv_len)
+    return packed
+
+
 def qk_indexmask_from_blockmax_cuda(blockmax, max_q, denom, q, k, thresh, blocksz=128, kv_len=0):
     """Key lists (the reference's form) from the block maxima: blocks that can hold a key, the sweep over
-    those blocks, the compaction."""
-    mask = qk_bitmask_from_blockmax_cuda(blockmax, max_q, denom, q, k, thresh, blocksz, kv_len)
-    return bitmask_to_indexmask_cuda(mask, kv_len or q.shape[2])
+    those blocks with its votes as bits, the key lists decoded from the bits."""
+    packed = qk_packedmask_from_blockmax_cuda(blockmax, max_q, denom, q, k, thresh, blocksz, kv_len)
+    return packedmask_to_indexmask_cuda(packed, kv_len or q.shape[2])
 
 
 def qk_indexmask_onepass_cuda(q, k, thresh, blocksz=128, kv_len=0):

@@ -105,7 +105,7 @@ def cached_attn_cuda(query, key, value, current_layer, ditrun, *args, **kwargs):
     pre-pass; on every other step: sparse attention from the cached lists (:95-114).
     The refresh step sweeps Q K^T once in full instead of twice (the dense pass also writes the score
     maximum of every row over every 64-key block, S*S/16 bytes per head, freed on return); the lists
-    are the same except for keys whose margin over the threshold is below fp32 rounding.  ``onepass=False`` runs the reference's sequence of two full sweeps."""
+    are the same.  ``onepass=False`` runs the reference's sequence of two full sweeps."""
     mask_cache = kwargs["mask_cache"]
     if mask_cache.run_fullattn(ditrun):
         if kwargs.get("onepass", True):
