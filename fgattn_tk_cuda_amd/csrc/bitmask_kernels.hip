@@ -50,9 +50,11 @@ __global__ __launch_bounds__(256) void pack_mask_kernel(uint32_t* __restrict__ p
       for (int u = 0; u < U; ++u) {
         uint32_t x = (cur[u][0] > 0 ? 1u : 0u) | (cur[u][1] > 0 ? 2u : 0u) | (cur[u][2] > 0 ? 4u : 0u) |
                      (cur[u][3] > 0 ? 8u : 0u);
-        x |= (uint32_t)__shfl_down((int)x, 1, 64) << 4;
-        x |= (uint32_t)__shfl_down((int)x, 2, 64) << 8;
-        x |= (uint32_t)__shfl_down((int)x, 4, 64) << 16;
+        // lanes l + 1, l + 2, l + 4 of the same 16-lane row (row_shl: data moves towards lane 0); only the
+        // lanes with l % 8 == 0 use the result, and their partners lie in their own group of eight
+        x |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x101, 0xf, 0xf, true) << 4;
+        x |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x102, 0xf, 0xf, true) << 8;
+        x |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x104, 0xf, 0xf, true) << 16;
         const int word = (c * SPAN + u * 256 + 4 * lane) >> 5;
         if ((lane & 7) == 0 && word < words_per_row) dst[word] = x;
       }
