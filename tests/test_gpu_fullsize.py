@@ -516,3 +516,24 @@ def test_reference_shape_75856_with_its_kv_length(dev):
             continue
         pp, den, _ = orc._softmax_rows(f32(q[0, h, r]) @ f32(k[0, h])[lst].T, 1.0 / np.sqrt(D), True)
         assert_close_o(f32(o3[0, h, r]), (pp @ f32(v[0, h])[lst]) / den[:, None], "sp_attn rows (%d,%d)" % (h, i))
+    # the same key lists through one full sweep: statistics with block maxima (8.6 GB at this shape), blocks
+    # a little below the threshold, the vote sweep over those blocks as bits, key lists from the bits
+    print("case reference shape 75856, one sweep", flush=True)
+    del o3
+    nb = Sp // 64
+    bmx = torch.empty((B, H, nb, Sp), device=dev)
+    mx1 = torch.full((B, H, 1, Sp), float("nan"), device=dev)
+    dn1 = torch.full((B, H, 1, Sp), float("nan"), device=dev)
+    capi.maxq_denom_blockmax(mx1, dn1, bmx, q, k, kv_len=kv)
+    assert torch.equal(mx1[..., :S], mx[..., :S]) and torch.equal(dn1[..., :S], dn[..., :S])
+    bi = torch.full((B, H, SB, nb), -1, dtype=torch.int32, device=dev)
+    bc = torch.zeros((B, H, SB), dtype=torch.int32, device=dev)
+    capi.blockmax_to_blocklists(bi, bc, bmx, mx, dn, thr * (1.0 - 1e-3), S, D, qblk=128, kv_len=kv)
+    del bmx
+    assert 0 < int(bc.sum()) < bc.numel() * orc.ceil_div(kv, 64)      # unclustered keys: most blocks hold a passing key
+    pk = torch.full((B, H, SB, Sp // 8), 0xA5, dtype=torch.uint8, device=dev)
+    capi.booleanmask_packed_blocks(pk, mx, dn, q, k, thr, bi, bc, qblk=128, kv_len=kv)
+    kvi1 = torch.full((B, H, SB, Sp), Sp, dtype=torch.int32, device=dev)
+    kvn1 = torch.zeros((B, H, SB), dtype=torch.int32, device=dev)
+    capi.packedmask_to_indexmask(kvi1, kvn1, pk, kv)
+    assert torch.equal(kvn1, kvn) and torch.equal(kvi1, kvi)
