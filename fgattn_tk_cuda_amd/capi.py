@@ -190,6 +190,12 @@ def sp_attn_blocks_balanced(o, q, k, v, blk_indices, blk_counts, *, lse=None, qb
                                                  qblk, B, H, S, D, kv_len, scale, _stream(stream)))
 
 
+def init():
+    """Sets up, on the current device, what a first call would otherwise set (the library's work-order
+    array, the dynamic-LDS limit of every attention kernel): afterwards every entry point only launches."""
+    _check(load().spattn_init())
+
+
 def qblock_order(order, counts, *, stream=None):
     """order: int32 [n] <- the q-blocks (flat indices of counts) longest list first; lists within
     a factor of two of each other keep the default order."""

@@ -910,13 +910,22 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
   }
 }
 
+// Raises the dynamic-LDS limit of one instantiation on the current device (once per device; the
+// launcher does it on the first launch, a caller that is about to record launches into a graph
+// does it beforehand through spattn_init).
+template <int D, int QBLK, int MODE, bool HAS_V, bool STATS>
+inline hipError_t prepare_attn_fwd() {
+  using Cfg = AttnCfg<D, MODE, HAS_V>;
+  static bool attr_set[kMaxDevices] = {};
+  return raise_lds_limit(reinterpret_cast<const void*>(attn_fwd_kernel<D, QBLK, MODE, HAS_V, STATS>), Cfg::kTotal, attr_set);
+}
+
 // Host launcher; returns hipError_t of the launch.
 template <int D, int QBLK, int MODE, bool HAS_V, bool STATS>
 inline hipError_t launch_attn_fwd(const AttnParams& p, hipStream_t stream) {
   using Cfg = AttnCfg<D, MODE, HAS_V>;
   auto kern = attn_fwd_kernel<D, QBLK, MODE, HAS_V, STATS>;
-  static bool attr_set[kMaxDevices] = {};
-  const hipError_t ea = raise_lds_limit(reinterpret_cast<const void*>(kern), Cfg::kTotal, attr_set);
+  const hipError_t ea = prepare_attn_fwd<D, QBLK, MODE, HAS_V, STATS>();
   if (ea != hipSuccess) return ea;
   const int total = p.nqblk * p.H * p.B;
   if (total <= 0) return hipSuccess;

@@ -12,4 +12,12 @@ hipError_t run_attn_blocks(const AttnParams& p, int D, int qblk, hipStream_t str
   return hipErrorInvalidValue;
 }
 
+hipError_t prepare_attn_blocks() {
+  hipError_t e = prepare_attn_fwd<128, 128, KV_BLOCKS, true, false>();
+  if (e == hipSuccess) e = prepare_attn_fwd<128, 64, KV_BLOCKS, true, false>();
+  if (e == hipSuccess) e = prepare_attn_fwd<64, 128, KV_BLOCKS, true, false>();
+  if (e == hipSuccess) e = prepare_attn_fwd<64, 64, KV_BLOCKS, true, false>();
+  return e;
+}
+
 }  // namespace spattn

@@ -17,4 +17,14 @@ hipError_t run_attn_dense(const AttnParams& p, int D, bool has_v, bool stats, hi
   return hipErrorInvalidValue;
 }
 
+hipError_t prepare_attn_dense() {
+  hipError_t e = prepare_attn_fwd<128, 128, KV_DENSE, true, false>();
+  if (e == hipSuccess) e = prepare_attn_fwd<128, 128, KV_DENSE, true, true>();
+  if (e == hipSuccess) e = prepare_attn_fwd<128, 128, KV_DENSE, false, true>();
+  if (e == hipSuccess) e = prepare_attn_fwd<64, 128, KV_DENSE, true, false>();
+  if (e == hipSuccess) e = prepare_attn_fwd<64, 128, KV_DENSE, true, true>();
+  if (e == hipSuccess) e = prepare_attn_fwd<64, 128, KV_DENSE, false, true>();
+  return e;
+}
+
 }  // namespace spattn

@@ -12,4 +12,12 @@ hipError_t run_attn_tokens(const AttnParams& p, int D, int qblk, hipStream_t str
   return hipErrorInvalidValue;
 }
 
+hipError_t prepare_attn_tokens() {
+  hipError_t e = prepare_attn_fwd<128, 128, KV_TOKENS, true, false>();
+  if (e == hipSuccess) e = prepare_attn_fwd<128, 64, KV_TOKENS, true, false>();
+  if (e == hipSuccess) e = prepare_attn_fwd<64, 128, KV_TOKENS, true, false>();
+  if (e == hipSuccess) e = prepare_attn_fwd<64, 64, KV_TOKENS, true, false>();
+  return e;
+}
+
 }  // namespace spattn

@@ -371,7 +371,12 @@ extern "C" {
 
 int spattn_init(void) {
   int* p = nullptr;
-  return done(scratch_on_current_device(&p));
+  if (int st = scratch_on_current_device(&p)) return done(st);
+  // what a first launch would otherwise set on this device: after this call every entry point only launches
+  hipError_t e = spattn::prepare_attn_dense();
+  if (e == hipSuccess) e = spattn::prepare_attn_blocks();
+  if (e == hipSuccess) e = spattn::prepare_attn_tokens();
+  return e == hipSuccess ? done(SPATTN_OK) : from_hip(e);
 }
 
 int spattn_sp_attn_blocks_balanced(void* o, float* lse, const void* q, const void* k, const void* v,

@@ -8,6 +8,10 @@ namespace spattn {
 hipError_t run_attn_tokens(const AttnParams& p, int D, int qblk, hipStream_t stream);
 hipError_t run_attn_blocks(const AttnParams& p, int D, int qblk, hipStream_t stream);
 hipError_t run_attn_dense(const AttnParams& p, int D, bool has_v, bool stats, hipStream_t stream);
+// every instantiation's dynamic-LDS limit on the current device (idempotent)
+hipError_t prepare_attn_tokens();
+hipError_t prepare_attn_blocks();
+hipError_t prepare_attn_dense();
 
 // mask_kernels.hip
 hipError_t run_booleanmask(void* out, int out_rows, float thresh, int mask_stride, const float* max_q,

@@ -241,8 +241,10 @@ int spattn_sp_attn_blocks_ordered(void* o, float* lse, const void* q, const void
  * q-blocks, else SPATTN_ERR_SCRATCH and nothing is launched.  All calls on one device share
  * that array: calls that overlap on one device (two streams, two threads) race on it - run
  * them one after the other, or use the _ordered form with a buffer per stream.
- * spattn_init looks the array's address up for the current device; optional, the first call
- * on a device does the same (call it before a graph capture starts). */
+ * spattn_init looks the array's address up for the current device and raises the dynamic-LDS limit
+ * of every attention kernel there - the two things a first call on a device otherwise does; it is
+ * optional, except that after it every entry point only launches kernels, which is what a caller
+ * needs who records his first calls on a device into a HIP graph. */
 int spattn_init(void);
 int spattn_sp_attn_blocks_balanced(void* o, float* lse, const void* q, const void* k, const void* v,
                                    const int* blk_indices, const int* blk_counts, int max_blocks, int qblk, int batch,

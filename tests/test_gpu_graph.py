@@ -3,6 +3,11 @@ replayed.  No entry point allocates, clears memory with a memset node or synchro
 cache-refresh step (statistics with block maxima -> lists -> attention) and the steady-state
 step are each capturable; every replay - with eager work and synchronisations between them -
 must reproduce the eager results bit for bit."""
+import os
+import subprocess
+import sys
+import textwrap
+
 import pytest
 import torch
 
@@ -95,3 +100,45 @@ def test_refresh_and_sparse_steps_replay_from_a_graph(dev, S, D):
         for name in buf:
             assert same(name), "replay %d: %s differs from the eager run" % (rep, name)
         assert torch.equal(eager.view(torch.int16), want["o_blk"].view(torch.int16))
+
+
+def test_capture_right_after_init_in_a_fresh_process(dev):
+    """A process whose first calls on the device are recorded into a graph: after spattn_init() no entry
+    point changes a device setting, so the capture needs no eager warm-up of the library."""
+    print("case graph capture after init", flush=True)
+    code = textwrap.dedent("""
+        import torch
+        from fgattn_tk_cuda_amd import capi, workloads as wl
+        dev = torch.device("cuda:0")
+        B, H, S, D, qblk = 1, 2, 1100, 128, 64
+        q, k, v = (t.to(dev) for t in wl.randn_qkv(B, H, S, D, seed=5))
+        nq = wl.ceil_div(S, qblk)
+        cnt = wl.zipf_counts(B, H, nq, s=1.2, lo=1, hi=wl.ceil_div(S, 64), seed=6)
+        bi, bc = (t.to(dev) for t in wl.ragged_block_lists(B, H, S, qblk, 64, cnt, seed=7))
+        o = torch.full_like(q, float("nan")); o2 = torch.full_like(q, float("nan")); od = torch.full_like(q, float("nan"))
+        mx = torch.empty((B, H, 1, 1152), device=dev); dn = torch.empty((B, H, 1, 1152), device=dev)
+        capi.init()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(g, stream=side):
+                capi.sp_attn_blocks(o, q, k, v, bi, bc, qblk=qblk)
+                capi.sp_attn_blocks_balanced(o2, q, k, v, bi, bc, qblk=qblk)
+                capi.fullattn_maxq_denom(od, mx, dn, q, k, v)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        e = torch.full_like(q, float("nan")); ed = torch.full_like(q, float("nan"))
+        capi.sp_attn_blocks(e, q, k, v, bi, bc, qblk=qblk)
+        capi.fullattn_maxq_denom(ed, mx, dn, q, k, v)
+        torch.cuda.synchronize()
+        assert torch.isfinite(e.float()).all()
+        assert torch.equal(o.view(torch.int16), e.view(torch.int16)) and torch.equal(o2.view(torch.int16), e.view(torch.int16))
+        assert torch.equal(od.view(torch.int16), ed.view(torch.int16))
+        print("captured-after-init ok")
+        """)
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=110,
+                       cwd=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    assert r.returncode == 0 and "captured-after-init ok" in r.stdout, r.stdout[-2000:] + r.stderr[-4000:]
