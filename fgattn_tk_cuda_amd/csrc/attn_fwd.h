@@ -62,8 +62,19 @@ struct AttnCfg {
   static constexpr int kLoadsPerTile = kTileBytes / 1024 / 4;   // per wave
 };
 
+// Waves per SIMD the register allocation aims at.  Two everywhere (256 registers), except for block lists at
+// d = 64 with 128-row q-blocks: that instantiation fits 168 registers with a handful of spills outside the
+// tile loop, its 40 KB ring lets three workgroups share a CU, and it is bound by the vector ALU, which a
+// third wave keeps fed (measured side by side on one board: -7 %; the dense and token-list forms of the same
+// shape need 40-50 spills for it and lose).
+template <int D, int QBLK, int MODE>
+constexpr int attn_waves_per_simd() {
+  return (D == 64 && QBLK == 128 && MODE == KV_BLOCKS) ? 3 : 2;
+}
+
 template <int D, int QBLK, int MODE, bool HAS_V, bool STATS>
-__global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnParams p) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(attn_waves_per_simd<D, QBLK, MODE>())))
+void attn_fwd_kernel(const AttnParams p) {
   static_assert(D == 64 || D == 128, "head dim");
   static_assert(QBLK == 64 || QBLK == 128, "q-block");
   using Cfg = AttnCfg<D, MODE, HAS_V>;
