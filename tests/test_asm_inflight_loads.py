@@ -9,7 +9,13 @@ names its destination registers.
 The HBM -> LDS copies set m0 inside their asm statement without telling the compiler (naming a
 reserved register as clobbered only draws a warning).  That is sound as long as the compiler
 itself never uses m0 in these kernels: the second check asserts that no instruction outside an
-asm statement names m0 in any translation unit that issues such copies."""
+asm statement names m0 in any translation unit that issues such copies.
+
+The tile loop of the attention kernels waits for its copies with hand-counted vmcnt values: that
+holds only while the compiler puts no vector-memory instruction of its own into the loop.  The
+third check finds the tile loop of every instantiation (one inner loop, closed by a branch back to
+its header) and asserts that it holds no scratch access (a spill) and no s_waitcnt vmcnt outside
+the asm statements (the compiler waiting for a load of its own)."""
 import re
 import shutil
 import subprocess
@@ -86,6 +92,50 @@ def m0_uses_outside_asm(listing):
     return found
 
 
+def tile_loop_findings(listing):
+    """{kernel: (scratch accesses, compiler vmcnt waits)} inside the tile loop of every attn_fwd_kernel
+    instantiation of a listing; a kernel whose loop is not found maps to None."""
+    out, name, cur = {}, None, []
+    for line in listing.split("\n"):
+        m = re.match(r"^(_ZN6spattn15attn_fwd_kernel\w+):", line)
+        if m:
+            name, cur = m.group(1), []
+        if name is None:
+            continue
+        cur.append(line)
+        if not line.startswith(".Lfunc_end"):
+            continue
+        hdr = next(((i, l.split(":")[0]) for i, l in enumerate(cur) if l.startswith(".LBB") and "Loop Header" in l), None)
+        last = None
+        if hdr is not None:
+            back = re.compile(r"s_c?branch\w*\s+" + re.escape(hdr[1]) + r"\b")
+            last = max((i for i in range(hdr[0], len(cur)) if back.match(cur[i].strip())), default=None)
+        if hdr is None or last is None:
+            out[name] = None
+        else:
+            scratch = waits = 0
+            inside = False
+            for l in cur[hdr[0]:last + 1]:
+                if "#ASMSTART" in l:
+                    inside = True
+                elif "#ASMEND" in l:
+                    inside = False
+                t = l.split(";")[0].strip()
+                scratch += t.startswith("scratch_")
+                waits += (not inside) and t.startswith("s_waitcnt") and "vmcnt" in t
+            out[name] = (scratch, waits)
+        name = None
+    return out
+
+
+def test_tile_loop_checker():
+    body = ("_ZN6spattn15attn_fwd_kernelILi64EEEvNS_10AttnParamsE:\n\ts_nop 0\n.LBB0_3:   ; =>This Inner Loop Header: Depth=1\n"
+            "\t;;#ASMSTART\n\ts_waitcnt vmcnt(4)\n\t;;#ASMEND\n%s\ts_cbranch_scc1 .LBB0_3\n\ts_endpgm\n.Lfunc_end0:\n")
+    assert tile_loop_findings(body % "") == {"_ZN6spattn15attn_fwd_kernelILi64EEEvNS_10AttnParamsE": (0, 0)}
+    assert list(tile_loop_findings(body % "\tscratch_load_dword v1, off, off\n\ts_waitcnt vmcnt(0)\n").values()) == [(1, 1)]
+    assert list(tile_loop_findings(body.replace("s_cbranch_scc1 .LBB0_3", "s_nop 1") % "").values()) == [None]
+
+
 def test_m0_checker_sees_a_compiler_use():
     ok = "\t;;#ASMSTART\n\ts_mov_b32 m0, s3\n\tglobal_load_lds_dwordx4 v1, s[0:1]\n\t;;#ASMEND\n\tv_mov_b32_e32 v2, v3\n"
     bad = ok + "\ts_mov_b32 m0, -1\n"
@@ -121,3 +171,7 @@ def test_no_instruction_touches_a_register_with_a_load_in_flight(tmp_path):
         assert "global_load_dword" in text, unit
         found = inflight_accesses(text)
         assert not found, "%s: %s" % (unit, found[:3])
+        loops = tile_loop_findings(text)
+        assert len(loops) >= 4, "%s: %d attention kernels found" % (unit, len(loops))
+        for kernel, f in loops.items():
+            assert f == (0, 0), "%s %s: tile loop not found, or scratch accesses / compiler vmcnt waits inside it: %s" % (unit, kernel, f)
