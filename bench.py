@@ -542,55 +542,6 @@ def cpu_baseline(res, budget_s=15.0):
     }
 
 
-def bench_lds_probe(dev, steps, warmup):
-    """LDS roofline of the attention tile loop (libspattn_probes.so): copies into LDS, K-operand
-    reads and V^T-operand reads, alone and in the mix of one 64-key tile of a 64-row q-block at
-    d = 128 (32 KB each per workgroup step), two workgroups of four waves per compute unit, no
-    matrix or vector work.  cfg3_floor_ms scales the time of a step to cfg 3's 425984 (q-block,
-    kv-block) pairs on the same 2 x CU workgroup slots."""
-    import ctypes
-
-    path = os.path.join(ROOT, "fgattn_tk_cuda_amd", "libspattn_probes.so")
-    lib = ctypes.CDLL(path)
-    f = lib.spattn_probe_lds_mix
-    f.restype = ctypes.c_int
-    f.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
-                  ctypes.POINTER(ctypes.c_float), ctypes.c_void_p]
-    src = torch.ones((1 << 20) + 65536, dtype=torch.uint8, device=dev)
-    sink = torch.zeros(4, dtype=torch.float32, device=dev)
-    cus = torch.cuda.get_device_properties(dev).multi_processor_count
-    nsteps, reps = 2000, 20
-    st = torch.cuda.current_stream().cuda_stream
-    names = {1: "copies", 2: "k_reads", 4: "v_reads", 8: "ds_write_b128", 3: "copies+k_reads", 5: "copies+v_reads",
-             6: "k_reads+v_reads", 7: "tile_mix", 23: "tile_mix_with_barrier"}
-    out = {"workgroups": 2 * cus, "steps_per_workgroup": nsteps, "kb_per_workgroup_step_and_kind": 32, "legs": {}}
-    for what, name in names.items():
-        ms = ctypes.c_float(0.0)
-        for _ in range(3):   # the first rounds raise the clocks
-            rc = f(what, src.data_ptr(), sink.data_ptr(), nsteps, reps, ctypes.byref(ms), st)
-            assert rc == 0, (name, rc)
-        kinds = bin(what & 15).count("1")
-        ns_step = ms.value * 1e6 / nsteps                   # one step of both workgroups of a compute unit
-        out["legs"][name] = {"ms": ms.value, "ns_per_step": ns_step,
-                             "gbps_per_cu": 2 * 32768 * kinds / ns_step,
-                             "cfg3_floor_ms": 425984.0 / (2 * cus) * ns_step * 1e-6}
-    # the gather of the headline launch with nothing else running (cfg 3 lists, real L2 hit rate)
-    B, H, S, D, nblk = 2, 32, 16384, 128, 26
-    _, k, v = (t.to(dev) for t in wl.randn_qkv(B, H, S, D, seed=0))
-    bi, _ = (t.to(dev) for t in wl.uniform_block_lists(B, H, S, 64, 64, nblk, seed=1))
-    g = lib.spattn_probe_copy_stream
-    g.restype = ctypes.c_int
-    g.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
-                  ctypes.POINTER(ctypes.c_float), ctypes.c_void_p]
-    ms = ctypes.c_float(0.0)
-    for _ in range(3):
-        rc = g(k.data_ptr(), v.data_ptr(), bi.data_ptr(), nblk, B * H, S, 50, ctypes.byref(ms), st)
-        assert rc == 0, rc
-    gathered = B * H * (S // 64) * nblk * 2 * 64 * D * 2
-    out["cfg3_copy_stream"] = {"ms": ms.value, "gathered_bytes": gathered, "tbps": gathered / ms.value / 1e9}
-    return out
-
-
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -598,7 +549,7 @@ def main(argv=None) -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-extras", action="store_true", help="only the headline kernel")
-    ap.add_argument("--only", default="", help="run one leg only: sparse|tokens|compact|dense|sweeps|copy|packed|topk|zipf|zipf64|cfg4|ldsprobe|gemm|blockmax (no JSON contract)")
+    ap.add_argument("--only", default="", help="run one leg only: sparse|tokens|compact|dense|sweeps|copy|packed|topk|zipf|zipf64|cfg4|gemm|blockmax (no JSON contract)")
     args = ap.parse_args(argv)
     if args.gpus != 1:
         print("bench.py: this library is single-GPU; run with --gpus 1 (got %d)" % args.gpus, file=sys.stderr)
@@ -613,7 +564,7 @@ def main(argv=None) -> int:
     if args.only:
         fn = {"sparse": bench_sparse, "compact": bench_compaction, "dense": bench_dense, "sweeps": bench_sweeps,
               "copy": bench_copy, "packed": bench_packed, "tokens": bench_tokens, "topk": bench_topk, "zipf": bench_zipf,
-              "zipf64": bench_zipf_sparse, "cfg4": bench_cfg4_end_to_end, "ldsprobe": bench_lds_probe, "gemm": bench_gemm, "blockmax": bench_blockmax}[args.only]
+              "zipf64": bench_zipf_sparse, "cfg4": bench_cfg4_end_to_end, "gemm": bench_gemm, "blockmax": bench_blockmax}[args.only]
         r = fn(dev, args.steps, args.warmup)
         r.pop("tensors", None)
         r.pop("step", None)

@@ -85,17 +85,6 @@ def build_lib(verbose: bool = True, poison: bool = False) -> Path:
     return out
 
 
-PROBES = PKG / "libspattn_probes.so"
-
-
-def build_probes(verbose: bool = True) -> Path:
-    """Compile the roofline probes (csrc/probes.hip) into libspattn_probes.so; bench.py --only ldsprobe runs them."""
-    _run([_hipcc(), *HIPCC_FLAGS, "-shared", "-o", str(PROBES), str(CSRC / "probes.hip")])
-    if verbose:
-        print("built", PROBES)
-    return PROBES
-
-
 def ext_path() -> Path:
     import sysconfig
 
@@ -137,7 +126,6 @@ def main(argv=None) -> int:
     build_lib()
     if not args.lib_only:
         build_torch_ext()
-        build_probes()
         build_lib(poison=True)
     return 0
 

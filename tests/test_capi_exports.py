@@ -76,16 +76,14 @@ def test_block_maxima_entry_points_check_their_arguments():
     assert lib.spattn_blockmax_to_blocklists(p16, p16, None, None, p16, p16, 0.5, 64, 1, 1, 128, 64, 0, 0.0, 2, None) == -1
 
 
-def test_debug_and_probe_libraries_load_and_export():
-    """The NaN-poisoning build exports the product library's whole surface; the probe library its two entry points."""
+def test_debug_library_loads_and_exports():
+    """The NaN-poisoning build exports the product library's whole surface."""
     from fgattn_tk_cuda_amd import build as bld
 
-    assert bld.POISON_LIB.exists() and bld.PROBES.exists(), "build them with `python -m fgattn_tk_cuda_amd.build`"
+    assert bld.POISON_LIB.exists(), "build them with `python -m fgattn_tk_cuda_amd.build`"
     poison = ctypes.CDLL(str(bld.POISON_LIB))
     for name in _declared():
         assert hasattr(poison, name), name
-    probes = ctypes.CDLL(str(bld.PROBES))
-    assert hasattr(probes, "spattn_probe_lds_mix") and hasattr(probes, "spattn_probe_copy_stream")
 
 
 def test_missing_library_is_an_error(monkeypatch, tmp_path):
