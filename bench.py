@@ -205,6 +205,58 @@ def _iid_mask(dev, seed):
     return (torch.rand((B, H, ms_ // 128, ms_), device=dev, generator=g) < c["keep"]).to(torch.int32)
 
 
+def bench_reference_sweep(dev, steps, warmup, seed=0):
+    """The reference's own sparse benchmark (python/benchmark.py:25-46): sp_attn with 128-row
+    q-blocks at d = 128, every q-block taking the same random permutation of the first
+    i * 4 * (S // 64) keys as its token list (python/spattn/mask_utils.py:191-203), i = 1..15, at
+    the smallest and the largest shape it loops over, (1,12,32760) and (1,40,75600).  The rows a
+    copy gathers are scattered 256-byte rows, not 64-row runs.  Per point: ms and TFLOP/s on the
+    kept keys (4 * S * keys * D flops per head)."""
+    D = 128
+    out = {"workload": "sp_attn, q-block 128, d=128, one random permutation of the first i*4*(S//64) keys per launch, "
+                       "shared by all q-blocks (the reference's python/benchmark.py sweep)", "shapes": {}}
+    g = torch.Generator(device=dev).manual_seed(seed + 77)
+    for (B, H, S) in ((1, 12, 32760), (1, 40, 75600)):
+        q, k, v = (torch.randn((B, H, S, D), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16) for _ in range(3))
+        Sp, SB = 128 * wl.ceil_div(S, 128), wl.ceil_div(S, 128)
+        o = torch.empty_like(q)
+        kvi = torch.empty((B, H, SB, Sp), dtype=torch.int32, device=dev)
+        kvn = torch.empty((B, H, SB), dtype=torch.int32, device=dev)
+        order = torch.empty((B * H * SB,), dtype=torch.int32, device=dev)
+        points = []
+        for i in range(1, 16):
+            keys = i * 4 * (S // 64)
+            row = torch.full((Sp,), Sp, dtype=torch.int32, device=dev)
+            row[:keys] = torch.randperm(keys, generator=g, device=dev).int()
+            kvi.copy_(row.expand(B, H, SB, Sp))
+            kvn.fill_(keys)
+            capi.qblock_order(order, kvn)
+
+            def step():
+                capi.sp_attn(o, q, k, v, kvi, kvn, qblk=128, order=order)
+
+            flops = 4.0 * B * H * S * keys * D
+            # about 0.3 s of launches per point behind two warm-up launches (the sweep has 30 points)
+            for _ in range(2):
+                step()
+            torch.cuda.synchronize()
+            est_ms = max(flops / 0.8e12, 0.05)
+            n = int(max(3, min(steps, 300.0 / est_ms)))
+            stream = torch.cuda.current_stream()
+            a, b_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record(stream)
+            for _ in range(n):
+                step()
+            b_.record(stream)
+            torch.cuda.synchronize()
+            ms = a.elapsed_time(b_) / n
+            points.append({"i": i, "keys": keys, "launches": n, "ms": ms, "tflops": flops / ms / 1e9,
+                           "mfma_frac": flops / ms / 1e9 / PEAK_BF16_TFLOPS})
+        out["shapes"]["%dx%dx%d" % (B, H, S)] = points
+        del q, k, v, o, kvi
+    return out
+
+
 def bench_compaction(dev, steps, warmup, seed=0, mask=None):
     """booleanmask_to_indexmask at the padded threshold workload: B=1, H=24, N=32760 -> mask
     [1,24,256,32768] int32.  mask: the vote mask of the threshold sweep (kept keys come in runs);
@@ -549,7 +601,7 @@ def main(argv=None) -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-extras", action="store_true", help="only the headline kernel")
-    ap.add_argument("--only", default="", help="run one leg only: sparse|tokens|compact|dense|sweeps|copy|packed|topk|zipf|zipf64|cfg4|gemm|blockmax (no JSON contract)")
+    ap.add_argument("--only", default="", help="run one leg only: sparse|tokens|compact|dense|sweeps|copy|packed|topk|zipf|zipf64|cfg4|gemm|blockmax|refsweep (no JSON contract)")
     args = ap.parse_args(argv)
     if args.gpus != 1:
         print("bench.py: this library is single-GPU; run with --gpus 1 (got %d)" % args.gpus, file=sys.stderr)
@@ -564,7 +616,8 @@ def main(argv=None) -> int:
     if args.only:
         fn = {"sparse": bench_sparse, "compact": bench_compaction, "dense": bench_dense, "sweeps": bench_sweeps,
               "copy": bench_copy, "packed": bench_packed, "tokens": bench_tokens, "topk": bench_topk, "zipf": bench_zipf,
-              "zipf64": bench_zipf_sparse, "cfg4": bench_cfg4_end_to_end, "gemm": bench_gemm, "blockmax": bench_blockmax}[args.only]
+              "zipf64": bench_zipf_sparse, "cfg4": bench_cfg4_end_to_end, "gemm": bench_gemm, "blockmax": bench_blockmax,
+              "refsweep": bench_reference_sweep}[args.only]
         r = fn(dev, args.steps, args.warmup)
         r.pop("tensors", None)
         r.pop("step", None)
@@ -652,6 +705,16 @@ def main(argv=None) -> int:
         out["topk_mask"] = {"workload": "cfg4 shape, q-block-mean top-k, %d keys per q-block" % tp["select_k"],
                             "ms": tp["ms"], "gbps": tp["bytes"] / tp["ms"] / 1e6,
                             "hbm_frac": tp["bytes"] / tp["ms"] / 1e6 / PEAK_HBM_GBPS, "algorithmic_bytes": tp["bytes"]}
+        ci = bench_compaction(dev, args.steps, args.warmup)
+        out["mask_pass_iid8"] = {"kernel": "compact_kernel (booleanmask_to_indexmask)",
+                                 "workload": "iid mask [1, 24, 256, 32768] int32 with 8 % of the keys set (the other reading of "
+                                             "cfg4's \"8 % kept\": 64 MB of indices written per launch)",
+                                 "ms": ci["ms"],
+                                 "roofline": {"bound": "hbm", "achieved": ci["bytes"] / ci["ms"] / 1e6, "peak": PEAK_HBM_GBPS,
+                                              "unit": "GB/s", "frac": ci["bytes"] / ci["ms"] / 1e6 / PEAK_HBM_GBPS,
+                                              "traffic": measured_traffic("compact_kernel_iid8"), "traffic_unit": "bytes",
+                                              "algorithmic_bytes": ci["bytes"]}}
+        out["reference_sweep"] = bench_reference_sweep(dev, args.steps, args.warmup)
         dn = bench_dense(dev, args.steps, args.warmup)
         out["dense_full_attn"] = {"workload": "cfg2: B=4 H=16 N=4096 d=64", "ms": dn["ms"],
                                   "tflops": dn["flops"] / (dn["ms"] * 1e-3) / 1e12,

@@ -297,15 +297,16 @@ void attn_fwd_kernel(const AttnParams p) {
   using G0 = std::integral_constant<int, 0>;
   using G1 = std::integral_constant<int, 1>;
   using G2 = std::integral_constant<int, 2>;
-  if (ntiles > 0) issue_tile(head_desc(0), kslot(0), false, G0{});
-  // The Q loads go out behind the copy of K0 and are counted by hand like the copies (a load
-  // the compiler sees makes it wait for every copy issued before the first use of Q): the wait
-  // for K0 covers them.  Rows past the end of the sequence read the last row and are zeroed.
+  // The Q loads go out first - their address does not wait for the list - and are counted by
+  // hand like the copies (a load the compiler sees makes it wait for every copy issued before
+  // the first use of Q): the wait for K0, issued behind them, covers them.  Rows past the end of
+  // the sequence read the last row and are zeroed.
   u32x4 qf[NT];
   {
     const uint16_t* qsrc = qh + (size_t)(qrow_ok ? qrow : p.S - 1) * D + 8 * g;
     load_q_uncounted<0, NT>(qf, qsrc);
   }
+  if (ntiles > 0) issue_tile(head_desc(0), kslot(0), false, G0{});
   int head_pending = 0;   // tile copies behind K0 when the first phase waits
   if (ntiles > 0) {
     if (1 < ntiles) { issue_tile(head_desc(1), kslot(1), false, G1{}); ++head_pending; }

@@ -9,7 +9,11 @@
 // returning (python/cuda_attn.cu:33-36 under -DNDEBUG).
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <ATen/hip/HIPGraphsUtils.cuh>
 #include <torch/extension.h>
+
+#include <mutex>
+#include <vector>
 
 #include "spattn_hip.h"
 
@@ -140,18 +144,70 @@ static void check_sp_attn_args(torch::Tensor& o, torch::Tensor& q, torch::Tensor
   TORCH_CHECK(kv_num_indices.numel() == q.size(0) * q.size(1) * kv_indices.size(2), "kv_num_indices must have B*H*SB entries");
 }
 
+// Work orders of the reference-named sp_attn, which has no argument to pass one in.  One entry per
+// (device, stream, address and size of the counts tensor); the entry remembers the version counter
+// of the counts it was computed from.  A call that finds its entry with the same version launches
+// the attention kernel and nothing else; a new version recomputes the order into the entry's buffer
+// (same stream, so launches that still read it are ahead in stream order); only the first sight of a
+// counts tensor allocates.  Buffers are never freed or handed to another key, so a launch recorded
+// into a graph keeps a valid pointer.  Any permutation of the q-blocks gives the same result: an
+// entry that outlived its counts tensor (same address, size and version by coincidence) can cost
+// balance, never correctness.
+struct OrderEntry {
+  int device;
+  void* stream;
+  const void* counts;
+  int64_t numel;
+  int64_t version;
+  torch::Tensor order;
+};
+static std::mutex g_order_mu;
+static std::vector<OrderEntry> g_orders;
+constexpr size_t kMaxOrderEntries = 1024;
+
+static int64_t counts_version(const torch::Tensor& t) {
+  return t.is_inference() ? 0 : (int64_t)t._version();
+}
+
+// The work order for these counts on the current stream; computes it if the cache has none.
+// Returns the tensor that owns the buffer (kept alive by the cache or, when the cache is full or
+// the stream is being captured into a graph, by the caller for the length of the call).
+static torch::Tensor cached_qblock_order(const torch::Tensor& counts) {
+  const int dev = (int)counts.device().index();
+  void* stream = cur_stream();
+  const int64_t ver = counts_version(counts);
+  auto compute = [&](torch::Tensor& order) {
+    check_status(spattn_qblock_order(order.data_ptr<int>(), counts.data_ptr<int>(), (int)counts.numel(), stream),
+                 "sp_attn (work order)");
+  };
+  const bool capturing =
+      c10::hip::currentStreamCaptureStatusMayInitCtx() != c10::hip::CaptureStatus::None;
+  std::lock_guard<std::mutex> lock(g_order_mu);
+  for (auto& e : g_orders) {
+    if (e.device == dev && e.stream == stream && e.counts == counts.data_ptr() && e.numel == counts.numel()) {
+      if (e.version != ver) {
+        compute(e.order);
+        e.version = ver;
+      }
+      return e.order;
+    }
+  }
+  torch::Tensor order = torch::empty({counts.numel()}, counts.options());
+  compute(order);
+  if (!capturing && g_orders.size() < kMaxOrderEntries)
+    g_orders.push_back(OrderEntry{dev, stream, counts.data_ptr(), counts.numel(), ver, order});
+  return order;
+}
+
 void sp_attn(torch::Tensor o, torch::Tensor q, torch::Tensor k, torch::Tensor v, torch::Tensor kv_indices,
              torch::Tensor kv_num_indices) {
   check_sp_attn_args(o, q, k, v, kv_indices, kv_num_indices);
   const DeviceGuard guard(q.device());
   // Threshold masks give lists of very different lengths: the q-blocks are handed to the
-  // workgroups longest list first (the order is a small device tensor from torch's caching
-  // allocator; lists within a factor of two of each other keep the default order).  Callers
-  // that reuse their lists compute the order once (qblock_order) and pass it to sp_attn_ex.
-  torch::Tensor order = torch::empty({kv_num_indices.numel()}, kv_num_indices.options());
-  check_status(spattn_qblock_order(order.data_ptr<int>(), kv_num_indices.data_ptr<int>(), (int)kv_num_indices.numel(),
-                                   cur_stream()),
-               "sp_attn (work order)");
+  // workgroups longest list first (lists within a factor of two of each other keep the default
+  // order).  The order is computed when the counts tensor is first seen or has been written to
+  // since (its version counter); every other call is the attention launch alone.
+  const torch::Tensor order = cached_qblock_order(kv_num_indices);
   sp_attn_impl(o, c10::nullopt, q, k, v, kv_indices, kv_num_indices, order.data_ptr<int>(), 0.0, 0);
 }
 

@@ -359,3 +359,72 @@ def test_functionals_with_mask_cache(dev):
     o3 = fn.attn_2xmask_cuda(q, k, v, 0, 0, blocksz=128)
     w3 = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float()[:, :, 0:2 * (S // 2):2], v.float()[:, :, 0:2 * (S // 2):2])
     assert_close_o(f32(o3), f32(w3), "attn_2xmask_cuda")
+
+
+def test_sp_attn_operator_keeps_its_work_order(dev):
+    """The reference-named operator has no argument for a work order: it computes one when it first sees a counts
+    tensor or when that tensor was written to since, and otherwise launches the attention kernel alone - no
+    allocation on repeated calls, the same bits as the C ABI, also after the counts changed in place and from a
+    recorded graph."""
+    print("case sp_attn operator work order", flush=True)
+    import fgattn_tk_cuda_amd.spattn.cuda_attn  # noqa: F401
+
+    ops = torch.ops.cuda_attn
+    B, H, S, D = 1, 3, 2048, 128
+    q, k, v = to_dev(dev, *wl.randn_qkv(B, H, S, D, seed=11))
+    g = torch.Generator().manual_seed(5)
+    SB, Sp = S // 128, S
+    kvi = torch.full((B, H, SB, Sp), Sp, dtype=torch.int32)
+    kvn = torch.zeros((B, H, SB), dtype=torch.int32)
+    for b in range(B):
+        for h in range(H):
+            for i in range(SB):
+                n = int(torch.randint(1, S // 2 if i % 3 else S, (1,), generator=g))   # very uneven lengths
+                kvi[b, h, i, :n] = torch.randperm(S, generator=g)[:n].sort().values.int()
+                kvn[b, h, i] = n
+    kvi, kvn = kvi.to(dev), kvn.to(dev)
+
+    def want_of(counts):
+        w = torch.full_like(q, float("nan"))
+        capi.sp_attn(w, q, k, v, kvi, counts, qblk=128)
+        return w
+
+    want = want_of(kvn)
+    o = torch.full_like(q, float("nan"))
+    ops.sp_attn(o, q, k, v, kvi, kvn)            # first sight of kvn: computes the order
+    torch.cuda.synchronize()
+    assert torch.equal(o, want)
+    n0 = torch.cuda.memory_stats(dev)["allocation.all.allocated"]
+    for _ in range(3):
+        o.fill_(float("nan"))
+        ops.sp_attn(o, q, k, v, kvi, kvn)
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_stats(dev)["allocation.all.allocated"] == n0, "repeated calls must not allocate"
+    assert torch.equal(o, want)
+    # the counts change in place (shorter lists): new order in the same buffer, same bits as the C ABI
+    kvn.copy_(torch.clamp(kvn // 3, min=1))
+    want2 = want_of(kvn)
+    n1 = torch.cuda.memory_stats(dev)["allocation.all.allocated"]
+    o.fill_(float("nan"))
+    ops.sp_attn(o, q, k, v, kvi, kvn)
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_stats(dev)["allocation.all.allocated"] == n1, "a new version of known counts must not allocate"
+    assert torch.equal(o, want2) and not torch.equal(want, want2)
+    # recorded into a graph after the order exists: replays reproduce the eager result
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        ops.sp_attn(o, q, k, v, kvi, kvn)         # this stream's own entry, made outside the capture
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        o.fill_(float("nan"))
+        with torch.cuda.graph(graph, stream=side):
+            ops.sp_attn(o, q, k, v, kvi, kvn)
+    torch.cuda.current_stream().wait_stream(side)
+    for rep in range(3):
+        o.fill_(float("nan"))
+        _ = (q.float() @ k.float().transpose(-1, -2)).sum()   # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(o, want2), "replay %d" % rep
