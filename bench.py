@@ -466,11 +466,11 @@ def bench_cfg4_end_to_end(dev, steps, warmup, seed=0):
     # routes 4 and 5: one sweep.  The statistics sweep also writes the score maximum of every row over
     # every 64-key block (1.6 GB); the threshold test runs on those maxima - no second Q K^T sweep.
     del pk
-    bmx = torch.empty((B, H, nb, Sp), dtype=torch.float32, device=dev)
+    bmx = torch.empty((B, H, nb, Sp), dtype=torch.bfloat16, device=dev)
     ms_fb, _ = time_steps(lambda: capi.fullattn_maxq_denom_blockmax(o, mx, dn, bmx, q, k, v), n_sw, 1)
     ms_mb, _ = time_steps(lambda: capi.maxq_denom_blockmax(mx, dn, bmx, q, k), n_sw, 1)
-    out["fullattn_maxq_denom_blockmax"] = {"ms": ms_fb, "blockmax_bytes": 4.0 * bmx.numel()}
-    out["maxq_denom_blockmax"] = {"ms": ms_mb, "blockmax_bytes": 4.0 * bmx.numel()}
+    out["fullattn_maxq_denom_blockmax"] = {"ms": ms_fb, "blockmax_bytes": 2.0 * bmx.numel()}
+    out["maxq_denom_blockmax"] = {"ms": ms_mb, "blockmax_bytes": 2.0 * bmx.numel()}
     for qblk in (128, 64):
         nq = wl.ceil_div(S, qblk)
         biq = torch.full((B, H, nq, nb), -1, dtype=torch.int32, device=dev)
@@ -482,7 +482,7 @@ def bench_cfg4_end_to_end(dev, steps, warmup, seed=0):
         ms_at, _ = time_steps(lambda: capi.sp_attn_blocks(o, q, k, v, biq, bcq, qblk=qblk, order=ordq), n_at, 2)
         fl = wl.kept_block_flops(kept, qblk, 64, D)
         # maxima of the blocks that hold a key, the two statistics rows, lists and counts
-        bl_bytes = 4.0 * B * H * nkb * S + 8.0 * B * H * S + 4.0 * kept + 4.0 * bcq.numel()
+        bl_bytes = 2.0 * B * H * nkb * S + 8.0 * B * H * S + 4.0 * kept + 4.0 * bcq.numel()
         out["blockmax%d" % qblk] = {
             "blockmax_to_blocklists_ms": ms_bl, "blockmax_to_blocklists_gbps": bl_bytes / ms_bl / 1e6,
             "blockmax_to_blocklists_hbm_frac": bl_bytes / ms_bl / 1e6 / PEAK_HBM_GBPS, "blockmax_to_blocklists_bytes": bl_bytes,
@@ -490,7 +490,9 @@ def bench_cfg4_end_to_end(dev, steps, warmup, seed=0):
             "sp_attn_blocks_ms": ms_at, "sp_attn_blocks_tflops": fl / ms_at / 1e9,
             "sp_attn_blocks_mfma_frac": fl / ms_at / 1e9 / PEAK_BF16_TFLOPS,
             "extra_sweep_ms": ms_mb - out["maxq_denom"]["ms"],
-            "prepass_plus_attention_ms": (ms_mb - out["maxq_denom"]["ms"]) + ms_bl + ms_order + ms_at}
+            "extra_sweep_ms_with_v": ms_fb - out["fullattn_maxq_denom"]["ms"],
+            "prepass_plus_attention_ms": (ms_mb - out["maxq_denom"]["ms"]) + ms_bl + ms_order + ms_at,
+            "cached_flow_after_dense_ms": (ms_fb - out["fullattn_maxq_denom"]["ms"]) + ms_bl + ms_order + ms_at}
     # route 6: the reference's key lists with one full sweep - block lists (128-row q-blocks) from the maxima,
     # then the threshold sweep over the kept blocks only, then the compaction as in route 1
     bi8 = torch.full((B, H, SB, nb), -1, dtype=torch.int32, device=dev)
@@ -513,7 +515,8 @@ def bench_cfg4_end_to_end(dev, steps, warmup, seed=0):
         "booleanmask_to_indexmask_ms": cp["ms"], "kept_keys": int(kvn2.sum().item()),
         "same_counts_as_two_sweeps": bool(torch.equal(kvn2, kvn)),
         "extra_sweep_ms": ms_mb - out["maxq_denom"]["ms"],
-        "prepass_plus_attention_ms": (ms_mb - out["maxq_denom"]["ms"]) + ms_bl8 + ms_sp + cp["ms"] + ms_order + ms_attn}
+        "prepass_plus_attention_ms": (ms_mb - out["maxq_denom"]["ms"]) + ms_bl8 + ms_sp + cp["ms"] + ms_order + ms_attn,
+        "cached_flow_after_dense_ms": (ms_fb - out["fullattn_maxq_denom"]["ms"]) + ms_bl8 + ms_sp + cp["ms"] + ms_order + ms_attn}
     # route 7: the same with the votes as bits (1/32 of the bytes) and the key lists decoded from the bits
     del mask
     pk8 = torch.empty((B, H, SB, Sp // 8), dtype=torch.uint8, device=dev)
@@ -525,7 +528,11 @@ def bench_cfg4_end_to_end(dev, steps, warmup, seed=0):
         "booleanmask_packed_blocks_ms": ms_pb, "booleanmask_packed_blocks_tflops": sp_flops / ms_pb / 1e9,
         "packedmask_to_indexmask_ms": ms_dec, "same_counts_as_two_sweeps": bool(torch.equal(kvn3, kvn)),
         "extra_sweep_ms": ms_mb - out["maxq_denom"]["ms"],
-        "prepass_plus_attention_ms": (ms_mb - out["maxq_denom"]["ms"]) + ms_bl8 + ms_pb + ms_dec + ms_order + ms_attn}
+        "extra_sweep_ms_with_v": ms_fb - out["fullattn_maxq_denom"]["ms"],
+        "prepass_plus_attention_ms": (ms_mb - out["maxq_denom"]["ms"]) + ms_bl8 + ms_pb + ms_dec + ms_order + ms_attn,
+        # what cached_attn_cuda adds behind the dense pass of a refresh step: the extra output of
+        # fullattn_maxq_denom_blockmax over fullattn_maxq_denom, then lists, restricted sweep, decode, order, attention
+        "cached_flow_after_dense_ms": (ms_fb - out["fullattn_maxq_denom"]["ms"]) + ms_bl8 + ms_pb + ms_dec + ms_order + ms_attn}
     assert torch.isfinite(o.float()).all().item(), "non-finite attention output"
     return out
 
@@ -541,16 +548,16 @@ def bench_blockmax(dev, steps, warmup, seed=0, tau=0.0102):
     nb, nkb = Sp // 64, wl.ceil_div(S, 64)
     mx = torch.empty((B, H, 1, Sp), device=dev)
     dn = torch.empty((B, H, 1, Sp), device=dev)
-    bmx = torch.empty((B, H, nb, Sp), dtype=torch.float32, device=dev)
+    bmx = torch.empty((B, H, nb, Sp), dtype=torch.bfloat16, device=dev)
     capi.maxq_denom_blockmax(mx, dn, bmx, q, k)
-    out = {"workload": "cfg4 block maxima fp32 [1,24,512,32768], threshold %g" % tau}
+    out = {"workload": "cfg4 block maxima bf16 [1,24,512,32768], threshold %g" % tau}
     for qblk in (128, 64):
         nq = wl.ceil_div(S, qblk)
         bi = torch.full((B, H, nq, nb), -1, dtype=torch.int32, device=dev)
         bc = torch.zeros((B, H, nq), dtype=torch.int32, device=dev)
         ms, _ = time_steps(lambda: capi.blockmax_to_blocklists(bi, bc, bmx, mx, dn, tau, S, D, qblk=qblk), steps, warmup)
         kept = int(bc.sum().item())
-        nbytes = 4.0 * B * H * nkb * S + 8.0 * B * H * S + 4.0 * kept + 4.0 * bc.numel()
+        nbytes = 2.0 * B * H * nkb * S + 8.0 * B * H * S + 4.0 * kept + 4.0 * bc.numel()
         out["q%d" % qblk] = {"ms": ms, "bytes": nbytes, "gbps": nbytes / ms / 1e6, "hbm_frac": nbytes / ms / 1e6 / PEAK_HBM_GBPS,
                              "kept_blocks": kept, "block_density": kept / (float(bc.numel()) * nkb)}
     return out
@@ -685,7 +692,7 @@ def main(argv=None) -> int:
                                          "algorithmic_bytes": tk4["booleanmask_to_indexmask_bytes"]}}
         bm4 = e2e["blockmax128"]
         out["mask_pass_block"] = {"kernel": "blockmax_to_blocklists_kernel<128> (threshold of the per-(row, key block) score maxima -> block lists)",
-                                  "workload": "cfg4 block maxima fp32 [1, 24, 512, 32768] of the statistics sweep, %.1f%% of the blocks kept"
+                                  "workload": "cfg4 block maxima bf16 [1, 24, 512, 32768] of the statistics sweep, %.1f%% of the blocks kept"
                                               % (100.0 * bm4["block_density"]),
                                   "ms": bm4["blockmax_to_blocklists_ms"],
                                   "roofline": {"bound": "hbm", "achieved": bm4["blockmax_to_blocklists_gbps"], "peak": PEAK_HBM_GBPS,

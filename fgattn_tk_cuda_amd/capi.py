@@ -326,16 +326,16 @@ def booleanmask_to_blocklists(blk_indices, blk_counts, booleanmask, seq, *, bloc
 def _need_blockmax(blockmax, B, H, S):
     sp = 128 * ((S + 127) // 128)
     if blockmax.numel() != B * H * (sp // 64) * sp:
-        raise ValueError("blockmax must be fp32 [B,H,%d,%d]" % (sp // 64, sp))
+        raise ValueError("blockmax must be bf16 [B,H,%d,%d]" % (sp // 64, sp))
 
 
 def maxq_denom_blockmax(max_q, denom, blockmax, q, k, *, kv_len=0, scale=0.0, stream=None):
-    """maxq_denom that also writes blockmax fp32 [B,H,Sp/64,Sp]: [J][r] = max of q[r].k[c] over the keys c < kv_len
+    """maxq_denom that also writes blockmax bf16 [B,H,Sp/64,Sp] (rounded toward +inf): [J][r] = max of q[r].k[c] over the keys c < kv_len
     of 64-key block J (blocks without such a key are left as they are)."""
     B, H, S, D = _bhsd(q)
     _need_padded(max_q, denom, B, H, S)
     _need_blockmax(blockmax, B, H, S)
-    _check(load().spattn_maxq_denom_blockmax(_ptr(max_q, f32), _ptr(denom, f32), _ptr(blockmax, f32), _ptr(q, bf16),
+    _check(load().spattn_maxq_denom_blockmax(_ptr(max_q, f32), _ptr(denom, f32), _ptr(blockmax, bf16), _ptr(q, bf16),
                                              _ptr(k, bf16), B, H, S, D, kv_len, scale, _stream(stream)))
 
 
@@ -345,7 +345,7 @@ def fullattn_maxq_denom_blockmax(o, max_q, denom, blockmax, q, k, v, *, kv_len=0
     _need_padded(max_q, denom, B, H, S)
     _need_blockmax(blockmax, B, H, S)
     _check(load().spattn_fullattn_maxq_denom_blockmax(_ptr(o, bf16), _ptr(max_q, f32), _ptr(denom, f32),
-                                                      _ptr(blockmax, f32), _ptr(q, bf16), _ptr(k, bf16), _ptr(v, bf16),
+                                                      _ptr(blockmax, bf16), _ptr(q, bf16), _ptr(k, bf16), _ptr(v, bf16),
                                                       B, H, S, D, kv_len, scale, _stream(stream)))
 
 
@@ -363,7 +363,7 @@ def blockmax_to_blocklists(blk_indices, blk_counts, blockmax, max_q, denom, thre
     _need_blockmax(blockmax, B, H, S)
     _blocklist_args(blk_indices, blk_counts, blockmask, B, H, SB, 128 * ((S + 127) // 128))
     _check(load().spattn_blockmax_to_blocklists(_ptr(blk_indices, i32), _ptr(blk_counts, i32),
-                                                _ptr(blockmask, torch.uint8), _ptr(blockmax, f32), _ptr(max_q, f32),
+                                                _ptr(blockmask, torch.uint8), _ptr(blockmax, bf16), _ptr(max_q, f32),
                                                 _ptr(denom, f32), float(threshold), int(qblk), B, H, S, int(D), kv_len,
                                                 scale, MB, _stream(stream)))
 

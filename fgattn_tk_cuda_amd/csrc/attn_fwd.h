@@ -443,7 +443,7 @@ void attn_fwd_kernel(const AttnParams p) {
   auto stat_finish = [&](float mloc, int tile) -> float {
     mloc = pair_max(mloc);
     if constexpr (STATS && KSPLIT == 1 && MODE == KV_DENSE) {
-      if (p.blockmax != nullptr && g == 0) p.blockmax[((size_t)bh * (p.Sp >> 6) + tile) * p.Sp + qrow] = mloc;
+      if (p.blockmax != nullptr && g == 0) p.blockmax[((size_t)bh * (p.Sp >> 6) + tile) * p.Sp + qrow] = bf16_round_up(mloc);
     }
     m_true = max_raw(m_true, mloc);
     return mloc * p.sf;

@@ -105,26 +105,30 @@ __global__ __launch_bounds__(256) void votes_to_blocklists_kernel(int* __restric
 }
 
 // Block maxima -> block lists: the threshold test of the mask pre-pass on the per-(row, key block)
-// score maxima that the statistics sweep writes next to max_q and denom (blockmax[b][h][J][r],
-// raw scores).  Some key c of block J passes  exp2((s[r,c] - max_q[r]) sf) / denom[r] > thresh
-// (include/mask_utils.cuh:231-238) exactly when the block's maximum does, so
+// score maxima that the statistics sweep writes next to max_q and denom (blockmax[b][h][J][r], raw
+// scores as bf16 rounded toward +inf: never below the true maximum).  Some key c of block J passes
+//   exp2((s[r,c] - max_q[r]) sf) / denom[r] > thresh      (include/mask_utils.cuh:231-238)
+// exactly when the block's maximum does, so
 //   MB[I, J] = OR_{r in q-block I, r < seq} ( blockmax[J][r] > t[r] ),
 //   t[r] = (log2 thresh + max_q[r] sf + log2 denom[r]) / sf   (the sweep kernel's per-row constant),
-// is the block mask of the threshold sweep without a second pass over Q K^T: one read of
-// 4 Sp Sp/64 bytes per head instead of 2 Sp^2 D flops.  One wave owns one q-block (QB rows, a lane
-// holds one or two of them); per key block a 256- or 512-byte line of maxima is compared and the
-// votes of the wave are one ballot; kept blocks are appended 64 at a time as in the kernels above.
+// holds every block of the threshold sweep's block mask - and, because of the rounding, possibly a
+// block whose maximum lies within one bf16 step (a factor 2^-8) below t[r] - without a second pass
+// over Q K^T: one read of 2 Sp Sp/64 bytes per head instead of 2 Sp^2 D flops.  One wave owns one
+// q-block.  A lane holds two neighbouring rows (one 32-bit load); with 128-row q-blocks a load
+// covers one key block, with 64-row q-blocks the two halves of the wave take two neighbouring key
+// blocks.  32 key blocks are in flight per step, the votes of a block are one ballot (or half of
+// one), kept blocks are appended 64 at a time as in the kernels above.
 template <int QB>
 __global__ __launch_bounds__(256) void blockmax_to_blocklists_kernel(int* __restrict__ blk_indices,
                                                                     int* __restrict__ blk_counts,
                                                                     unsigned char* __restrict__ blockmask,
-                                                                    const float* __restrict__ blockmax,
+                                                                    const uint16_t* __restrict__ blockmax,
                                                                     const float* __restrict__ max_q,
                                                                     const float* __restrict__ denom, float log2_thresh,
                                                                     float sf, int heads_total, int S, int Sp, int kv_len,
                                                                     int max_blocks, int bm_stride) {
-  constexpr int RPL = QB / 64;   // rows per lane
-  constexpr int U = 16;          // key blocks in flight per wave
+  constexpr int BPL = 128 / QB;  // key blocks per load instruction (1 or 2)
+  constexpr int U = 32 / BPL;    // loads in flight per wave: 32 key blocks per step
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int nqb = (S + QB - 1) / QB;
@@ -132,42 +136,48 @@ __global__ __launch_bounds__(256) void blockmax_to_blocklists_kernel(int* __rest
   const int nblk = (kv_len + 63) >> 6;    // key blocks that hold a key
   const int nbs = Sp >> 6;                // block rows of a head in blockmax
   const float inv_sf = 1.f / sf;
+  const int rl = (QB == 128) ? lane : (lane & 31);   // this lane's row pair within the q-block
+  const int jl = (QB == 128) ? 0 : (lane >> 5);      // this lane's key block within a load
   for (int row = blockIdx.x * 4 + wave; row < rows; row += gridDim.x * 4) {
     const int bh = row / nqb, I = row - bh * nqb;
-    float t[RPL];
-    int r[RPL];
+    const int r0 = I * QB + 2 * rl;       // rows r0, r0 + 1 (Sp is even: both inside the padded row)
+    float t[2];
 #pragma unroll
-    for (int j = 0; j < RPL; ++j) {
-      r[j] = I * QB + 64 * j + lane;
+    for (int j = 0; j < 2; ++j) {
       t[j] = __builtin_huge_valf();   // a row that does not exist, or has no key, never votes
-      if (r[j] < S) {
-        const float mq = max_q[(size_t)bh * Sp + r[j]];
-        const float dn = denom[(size_t)bh * Sp + r[j]];
+      if (r0 + j < S) {
+        const float mq = max_q[(size_t)bh * Sp + r0 + j];
+        const float dn = denom[(size_t)bh * Sp + r0 + j];
         if (dn > 0.f) t[j] = (log2_thresh + (mq * sf + __log2f(dn))) * inv_sf;
       }
-      r[j] = r[j] < Sp ? r[j] : Sp - 1;
     }
-    const float* __restrict__ src = blockmax + (size_t)bh * nbs * Sp;
+    const uint16_t* __restrict__ src = blockmax + (size_t)bh * nbs * Sp + r0;
     int* __restrict__ dst = blk_indices + (size_t)row * max_blocks;
     unsigned char* mrow = blockmask ? blockmask + (size_t)row * bm_stride : nullptr;
     int count = 0;
     for (int J0 = 0; J0 < nblk; J0 += 64) {
       unsigned long long word = 0;   // bit j: block J0 + j is kept
 #pragma unroll 1
-      for (int u0 = 0; u0 < 64 && J0 + u0 < nblk; u0 += U) {
-        float x[U][RPL];
+      for (int u0 = 0; u0 < 64 && J0 + u0 < nblk; u0 += 32) {
+        uint32_t x[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-          const int J = J0 + u0 + u;
+          const int J = J0 + u0 + BPL * u + jl;
           const int Jc = J < nblk ? J : nblk - 1;
-#pragma unroll
-          for (int j = 0; j < RPL; ++j) x[u][j] = __builtin_nontemporal_load(src + (size_t)Jc * Sp + r[j]);
+          x[u] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(src + (size_t)Jc * Sp));
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-          bool f = x[u][0] > t[0];
-          if constexpr (RPL == 2) f = f || (x[u][1] > t[1]);
-          if (__ballot(f) != 0ull && J0 + u0 + u < nblk) word |= 1ull << (u0 + u);
+          const float lo = __builtin_bit_cast(float, x[u] << 16);
+          const float hi = __builtin_bit_cast(float, x[u] & 0xffff0000u);
+          const unsigned long long b = __ballot(lo > t[0] || hi > t[1]);
+          const int J = J0 + u0 + BPL * u;
+          if constexpr (BPL == 1) {
+            if (b != 0ull && J < nblk) word |= 1ull << (u0 + u);
+          } else {
+            if ((uint32_t)b != 0u && J < nblk) word |= 1ull << (u0 + 2 * u);
+            if ((uint32_t)(b >> 32) != 0u && J + 1 < nblk) word |= 1ull << (u0 + 2 * u + 1);
+          }
         }
       }
       append_blocks((word >> lane) & 1ull, J0 + lane, bm_stride, count, dst, mrow, max_blocks);
@@ -200,7 +210,7 @@ hipError_t run_votes_to_blocklists(int* blk_indices, int* blk_counts, unsigned c
   return hipGetLastError();
 }
 
-hipError_t run_blockmax_to_blocklists(int* blk_indices, int* blk_counts, unsigned char* blockmask, const float* blockmax,
+hipError_t run_blockmax_to_blocklists(int* blk_indices, int* blk_counts, unsigned char* blockmask, const uint16_t* blockmax,
                                       const float* max_q, const float* denom, float thresh, float sf, int qblk,
                                       int heads_total, int S, int kv_len, int max_blocks, hipStream_t stream) {
   const int nqb = (S + qblk - 1) / qblk;

@@ -123,7 +123,7 @@ int spattn_maxq_denom(float* max_q, float* denom, const void* q, const void* k, 
   return from_hip(spattn::run_attn_dense(p, D, false, true, as_stream(stream)));
 }
 
-int spattn_fullattn_maxq_denom_blockmax(void* o, float* max_q, float* denom, float* blockmax, const void* q, const void* k,
+int spattn_fullattn_maxq_denom_blockmax(void* o, float* max_q, float* denom, void* blockmax, const void* q, const void* k,
                                         const void* v, int B, int H, int S, int D, int kv_len, float scale, void* stream) {
   if (int st = check_qkv(q, k, B, H, S, D)) return done(st);
   if (!o || !v || !max_q || !denom || !blockmax) return done(SPATTN_ERR_NULL);
@@ -131,31 +131,33 @@ int spattn_fullattn_maxq_denom_blockmax(void* o, float* max_q, float* denom, flo
   spattn::AttnParams p = base_params(q, k, v, o, B, H, S, D, kv_len, scale, 128);
   p.max_q = max_q;
   p.denom = denom;
-  p.blockmax = blockmax;
+  p.blockmax = static_cast<uint16_t*>(blockmax);
   return from_hip(spattn::run_attn_dense(p, D, true, true, as_stream(stream)));
 }
 
-int spattn_maxq_denom_blockmax(float* max_q, float* denom, float* blockmax, const void* q, const void* k, int B, int H,
+int spattn_maxq_denom_blockmax(float* max_q, float* denom, void* blockmax, const void* q, const void* k, int B, int H,
                                int S, int D, int kv_len, float scale, void* stream) {
   if (int st = check_qkv(q, k, B, H, S, D)) return done(st);
   if (!max_q || !denom || !blockmax) return done(SPATTN_ERR_NULL);
   spattn::AttnParams p = base_params(q, k, nullptr, nullptr, B, H, S, D, kv_len, scale, 128);
   p.max_q = max_q;
   p.denom = denom;
-  p.blockmax = blockmax;
+  p.blockmax = static_cast<uint16_t*>(blockmax);
   return from_hip(spattn::run_attn_dense(p, D, false, true, as_stream(stream)));
 }
 
-int spattn_blockmax_to_blocklists(int* blk_indices, int* blk_counts, void* blockmask, const float* blockmax,
+int spattn_blockmax_to_blocklists(int* blk_indices, int* blk_counts, void* blockmask, const void* blockmax,
                                   const float* max_q, const float* denom, float threshold, int qblk, int B, int H, int S,
                                   int D, int kv_len, float scale, int max_blocks, void* stream) {
   if (!blk_indices || !blk_counts || !blockmax || !max_q || !denom) return done(SPATTN_ERR_NULL);
+  if (misaligned(blockmax)) return done(SPATTN_ERR_ALIGN);
   if (D != 64 && D != 128) return done(SPATTN_ERR_HEAD_DIM);
   if (B <= 0 || H <= 0 || S <= 0 || S >= (1 << 24) || max_blocks <= 0) return done(SPATTN_ERR_SHAPE);
   if (qblk != 64 && qblk != 128) return done(SPATTN_ERR_QBLK);
   const int kv = (kv_len <= 0 || kv_len > S) ? S : kv_len;
   const float sc = scale > 0.f ? scale : 1.0f / sqrtf((float)D);
-  return from_hip(spattn::run_blockmax_to_blocklists(blk_indices, blk_counts, static_cast<unsigned char*>(blockmask), blockmax,
+  return from_hip(spattn::run_blockmax_to_blocklists(blk_indices, blk_counts, static_cast<unsigned char*>(blockmask),
+                                                     static_cast<const uint16_t*>(blockmax),
                                                      max_q, denom, threshold, spattn::kLog2e * sc, qblk, B * H, S, kv,
                                                      max_blocks, as_stream(stream)));
 }

@@ -32,7 +32,7 @@ struct AttnParams {
   float* lse;         // optional fp32 [B,H,S], natural log
   float* max_q;       // optional fp32 [B,H,1,Sp], raw (unscaled) row max
   float* denom;       // optional fp32 [B,H,1,Sp]
-  float* blockmax;    // optional fp32 [B,H,Sp/64,Sp]: raw max of row r over the keys of block J at [J][r] (dense + statistics only)
+  uint16_t* blockmax; // optional bf16 [B,H,Sp/64,Sp]: raw max of row r over the keys of block J at [J][r], rounded toward +inf (dense + statistics only)
   const int* idx;     // [B,H,SBq,idx_stride] token ids or block ids
   const int* cnt;     // [B*H*SBq]
   int idx_stride;
@@ -53,6 +53,13 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
   f32x2 f = {lo, hi};
   bf16x2 b = __builtin_convertvector(f, bf16x2);   // v_cvt_pk_bf16_f32, round to nearest even
   return __builtin_bit_cast(uint32_t, b);
+}
+
+// The smallest bf16 that is not below x (x not NaN): negative values are truncated, positive ones
+// rounded away from zero; -inf stays -inf.
+__device__ __forceinline__ uint16_t bf16_round_up(float x) {
+  const uint32_t b = __builtin_bit_cast(uint32_t, x);
+  return (uint16_t)((b + ((b >> 31) ? 0u : 0xffffu)) >> 16);
 }
 
 // Largest of three floats in one instruction.  Written as asm: through fmaxf the compiler first

@@ -33,7 +33,7 @@ hipError_t run_packed_to_blocklists(int* blk_indices, int* blk_counts, unsigned 
 hipError_t run_votes_to_blocklists(int* blk_indices, int* blk_counts, unsigned char* blockmask, const int* votes,
                                    int rows, int mask_stride, int kv_len, int max_blocks, hipStream_t stream);
 
-hipError_t run_blockmax_to_blocklists(int* blk_indices, int* blk_counts, unsigned char* blockmask, const float* blockmax,
+hipError_t run_blockmax_to_blocklists(int* blk_indices, int* blk_counts, unsigned char* blockmask, const uint16_t* blockmax,
                                       const float* max_q, const float* denom, float thresh, float sf, int qblk,
                                       int heads_total, int S, int kv_len, int max_blocks, hipStream_t stream);
 

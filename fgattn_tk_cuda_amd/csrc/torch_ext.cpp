@@ -311,9 +311,9 @@ void maxq_denom(torch::Tensor o_max_q, torch::Tensor o_denom, torch::Tensor q, t
 // threshold test on those maxima: the block-level form of booleanmask_128 + booleanmask_to_indexmask
 // (python/extension.cpp:229-340) that needs no second sweep over Q K^T.
 void check_blockmax(const torch::Tensor& blockmax, const torch::Tensor& q_like, int64_t B, int64_t H, int64_t S) {
-  check_aux(blockmax, "blockmax", at::kFloat, q_like);
+  check_aux(blockmax, "blockmax", at::kBFloat16, q_like);
   const int64_t sp = padded128(S);
-  TORCH_CHECK(blockmax.numel() == B * H * (sp / 64) * sp, "blockmax must be fp32 [B,H,Sp/64,Sp] with Sp = 128*ceil(S/128)");
+  TORCH_CHECK(blockmax.numel() == B * H * (sp / 64) * sp, "blockmax must be bf16 [B,H,Sp/64,Sp] with Sp = 128*ceil(S/128)");
 }
 
 void fullattn_maxq_denom_blockmax(torch::Tensor o, torch::Tensor o_max_q, torch::Tensor o_denom, torch::Tensor blockmax,
@@ -329,7 +329,7 @@ void fullattn_maxq_denom_blockmax(torch::Tensor o, torch::Tensor o_max_q, torch:
   check_blockmax(blockmax, q, q.size(0), q.size(1), q.size(2));
   const DeviceGuard guard(q.device());
   check_status(spattn_fullattn_maxq_denom_blockmax(o.data_ptr(), o_max_q.data_ptr<float>(), o_denom.data_ptr<float>(),
-                                                   blockmax.data_ptr<float>(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                                   blockmax.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
                                                    (int)q.size(0), (int)q.size(1), (int)q.size(2), (int)q.size(3),
                                                    checked_kv_len(kv_len, q), (float)scale, cur_stream()),
                "fullattn_maxq_denom_blockmax");
@@ -345,7 +345,7 @@ void maxq_denom_blockmax(torch::Tensor o_max_q, torch::Tensor o_denom, torch::Te
   TORCH_CHECK(o_max_q.numel() == need && o_denom.numel() == need, "o_max_q / o_denom must be [B,H,1,128*ceil(S/128)]");
   check_blockmax(blockmax, q, q.size(0), q.size(1), q.size(2));
   const DeviceGuard guard(q.device());
-  check_status(spattn_maxq_denom_blockmax(o_max_q.data_ptr<float>(), o_denom.data_ptr<float>(), blockmax.data_ptr<float>(),
+  check_status(spattn_maxq_denom_blockmax(o_max_q.data_ptr<float>(), o_denom.data_ptr<float>(), blockmax.data_ptr(),
                                           q.data_ptr(), k.data_ptr(), (int)q.size(0), (int)q.size(1), (int)q.size(2),
                                           (int)q.size(3), checked_kv_len(kv_len, q), (float)scale, cur_stream()),
                "maxq_denom_blockmax");
@@ -375,7 +375,7 @@ void blockmax_to_blocklists(torch::Tensor blk_idx, torch::Tensor blk_cnt, OptTen
     bm = blockmask->data_ptr();
   }
   const DeviceGuard guard(blk_idx.device());
-  check_status(spattn_blockmax_to_blocklists(blk_idx.data_ptr<int>(), blk_cnt.data_ptr<int>(), bm, blockmax.data_ptr<float>(),
+  check_status(spattn_blockmax_to_blocklists(blk_idx.data_ptr<int>(), blk_cnt.data_ptr<int>(), bm, blockmax.data_ptr(),
                                              o_max_q.data_ptr<float>(), o_denom.data_ptr<float>(), (float)threshold, (int)qblk,
                                              (int)B, (int)H, (int)seq, (int)head_dim, (int)kv_len, (float)scale,
                                              (int)blk_idx.size(3), cur_stream()),

@@ -86,17 +86,23 @@ class CompressMaskCache(NaiveMaskCache):
         kv_indices, counts = packedmask_to_indexmask_cuda(packed, seq_len)
         return kv_indices, counts.view_as(kv_num_indices)
 
-    def update_cache(self, layer, kv_indices, kv_num_indices):
+    def update_cache(self, layer, kv_indices, kv_num_indices, seq_len=None):
+        """seq_len: the number of keys the ids range over, rounded up to a multiple of 128 for the bit
+        rows; default: the width of the lists, which is right for lists as wide as the sequence (what
+        the threshold pre-pass returns).  Narrower lists (top-k) need it; an id that does not fit is an
+        error, not a dropped key."""
         B, H, SB, stride = kv_indices.shape
+        width = _padded(int(seq_len)) if seq_len is not None else int(stride)
         pos = torch.arange(stride, device=kv_indices.device).view(1, 1, 1, stride)
-        live = (pos < kv_num_indices.reshape(B, H, SB, 1)) & (kv_indices >= 0) & (kv_indices < stride)
-        votes = torch.zeros((B, H, SB, stride + 1), dtype=torch.int32, device=kv_indices.device)
-        # entries behind the count (or outside the row) are sent to a spare column
-        votes.scatter_(3, torch.where(live, kv_indices, torch.full_like(kv_indices, stride)).long(), 1)
-        votes = votes[..., :stride].contiguous()
-        seq_len = int(stride)
-        packed = pack_votes_cuda(votes) if votes.is_cuda and stride % 128 == 0 else pack(votes > 0)
-        self.cache[layer] = (packed, seq_len, kv_num_indices)
+        live = (pos < kv_num_indices.reshape(B, H, SB, 1)) & (kv_indices >= 0)
+        if bool((live & (kv_indices >= width)).any()):
+            raise ValueError("CompressMaskCache: a listed key id does not fit %d keys; pass seq_len" % width)
+        votes = torch.zeros((B, H, SB, width + 1), dtype=torch.int32, device=kv_indices.device)
+        # entries behind the count are sent to a spare column
+        votes.scatter_(3, torch.where(live, kv_indices, torch.full_like(kv_indices, width)).long(), 1)
+        votes = votes[..., :width].contiguous()
+        packed = pack_votes_cuda(votes) if votes.is_cuda and width % 128 == 0 else pack(votes > 0)
+        self.cache[layer] = (packed, width, kv_num_indices)
         self.order[layer] = qblock_order_cuda(kv_num_indices) if _is_dev(kv_num_indices) else None
 
 
@@ -369,11 +375,37 @@ def qk_blocklists_cuda(q, k, thresh, qblk=128, kv_len=0):
     return qk_blocklists_from_maxq_denom_cuda(max_q, denom, q, k, thresh, qblk, kv_len)
 
 
-def blockmax_buffer(q):
-    """fp32 [B,H,Sp/64,Sp] for the per-(row, key block) score maxima of a statistics sweep."""
+# Largest block-maxima buffer the one-sweep routes allocate without being told to (bytes).  The
+# buffer takes 2 * Sp * Sp / 64 bytes per head: 0.81 GB at (1,24,32768), 1.5 GB at (1,12,75648),
+# 4.3 GB at (1,24,75904), 7.2 GB at (1,40,75648).  Above the budget the callers fall back to the
+# reference's two full sweeps, which need no such buffer.
+BLOCKMAX_BUDGET_BYTES = 2 << 30
+
+
+def blockmax_bytes(q):
+    """Bytes of the block-maxima buffer for a statistics sweep over q [B,H,S,D]."""
     B, H, S, _ = q.shape
     sp = _padded(S)
-    return torch.empty((B, H, sp // KVBLK, sp), dtype=torch.float32, device=q.device)
+    return 2 * B * H * (sp // KVBLK) * sp
+
+
+def use_onepass(q, onepass=None, budget_bytes=None):
+    """Whether a refresh step takes the one-sweep route (statistics sweep with block maxima, then the
+    threshold on those) or the reference's two full sweeps.  onepass True / False decides outright;
+    None decides by the size of the block-maxima buffer against budget_bytes (default
+    BLOCKMAX_BUDGET_BYTES)."""
+    if onepass is not None:
+        return bool(onepass)
+    budget = BLOCKMAX_BUDGET_BYTES if budget_bytes is None else int(budget_bytes)
+    return blockmax_bytes(q) <= budget
+
+
+def blockmax_buffer(q):
+    """bf16 [B,H,Sp/64,Sp] for the per-(row, key block) score maxima of a statistics sweep (the
+    sweep rounds them toward +inf)."""
+    B, H, S, _ = q.shape
+    sp = _padded(S)
+    return torch.empty((B, H, sp // KVBLK, sp), dtype=torch.bfloat16, device=q.device)
 
 
 def blockmax_to_blocklists_cuda(blockmax, max_q, denom, thresh, seq, head_dim, qblk=128, kv_len=0, max_blocks=None,
@@ -394,8 +426,9 @@ def blockmax_to_blocklists_cuda(blockmax, max_q, denom, thresh, seq, head_dim, q
 
 def qk_blocklists_onepass_cuda(q, k, thresh, qblk=128, kv_len=0):
     """KV-block lists from ONE sweep over Q K^T: the statistics sweep also writes the maximum of
-    every row over every 64-key block, and the threshold test runs on those maxima.  Same lists as
-    qk_blocklists_cuda except where a block's best key sits within rounding of the threshold."""
+    every row over every 64-key block (as bf16, rounded up), and the threshold test runs on those
+    maxima.  The lists hold every block of qk_blocklists_cuda's and possibly a block whose best key
+    misses the threshold by less than one bf16 step (2^-8) of its raw score."""
     max_q, denom = _stats_buffers(q)
     blockmax = blockmax_buffer(q)
     spattn_interface.maxq_denom_blockmax(max_q, denom, blockmax, q.contiguous(), k.contiguous(), 0.0, kv_len)
@@ -403,10 +436,12 @@ def qk_blocklists_onepass_cuda(q, k, thresh, qblk=128, kv_len=0):
 
 
 # The key-list route thresholds the block maxima a little below the vote threshold: the statistics
-# sweep and the vote sweep round a score differently (one rounds s and compares, the other accumulates
-# s - t in the matrix unit), so a key whose margin is within that rounding could otherwise sit in a block
-# the maxima leave out.  tau (1 - 1e-3) moves the block test by about 0.01 raw score units, a hundred times
-# the rounding of either sweep; the few blocks it adds contribute zero votes.
+# sweep and the vote sweep round a score differently in fp32 (one rounds s and compares, the other
+# accumulates s - t in the matrix unit), so a key whose margin is within that rounding could otherwise
+# sit in a block the maxima leave out.  Two margins cover it: the stored maxima are rounded UP to bf16
+# (up to 2^-8 of the score's own magnitude, so the margin grows with the scores), and tau (1 - 1e-3)
+# moves the block test by about 0.01 raw score units whatever the magnitude.  The blocks either adds
+# contribute zero votes.
 _BLOCK_THRESH_SLACK = 1.0 - 1e-3
 
 

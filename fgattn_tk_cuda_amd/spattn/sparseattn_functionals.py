@@ -103,12 +103,16 @@ def sparse_attn_from_cache_cuda(query, key, value, *args, **kwargs):
 def cached_attn_cuda(query, key, value, current_layer, ditrun, *args, **kwargs):
     """On the steps that refresh the cache: dense attention with statistics, then the mask
     pre-pass; on every other step: sparse attention from the cached lists (:95-114).
-    The refresh step sweeps Q K^T once in full instead of twice (the dense pass also writes the score
-    maximum of every row over every 64-key block, S*S/16 bytes per head, freed on return); the lists
-    are the same.  ``onepass=False`` runs the reference's sequence of two full sweeps."""
+    Where the buffer for it fits the budget, the refresh step sweeps Q K^T once in full instead of
+    twice: the dense pass also writes the score maximum of every row over every 64-key block (bf16,
+    S*S/32 bytes per head, freed on return) and the threshold sweep then runs over the key blocks that
+    can hold a key only; the lists are the same.  ``onepass=True`` / ``False`` forces one route
+    (False: the reference's two full sweeps, no extra buffer); by default the route is the one-sweep
+    one when the buffer is at most ``blockmax_budget_bytes`` (default
+    ``mask_utils.BLOCKMAX_BUDGET_BYTES``, 2 GiB)."""
     mask_cache = kwargs["mask_cache"]
     if mask_cache.run_fullattn(ditrun):
-        if kwargs.get("onepass", True):
+        if mask_utils.use_onepass(query, kwargs.get("onepass"), kwargs.get("blockmax_budget_bytes")):
             # the dense pass also writes the block maxima; the threshold sweep then runs over the key
             # blocks that can hold a key only
             out = _out_like(query)
@@ -118,9 +122,11 @@ def cached_attn_cuda(query, key, value, current_layer, ditrun, *args, **kwargs):
             kv_indices, kv_num_indices = mask_utils.qk_indexmask_from_blockmax_cuda(
                 blockmax, max_q, denom, query, key, kwargs["thresh"], blocksz=kwargs["blocksz"])
         else:
+            # the reference's two full sweeps; the votes of the second leave it as bits (1/32 of the
+            # int32 mask of python/spattn/mask_utils.py:358-382, the same lists)
             out, max_q, denom = _dense_with_stats(query, key, value)
-            kv_indices, kv_num_indices = mask_utils.qk_indexmask_from_maxq_denom_cuda(
-                max_q, denom, query, key, kwargs["thresh"], blocksz=kwargs["blocksz"])
+            packed = mask_utils.qk_packedmask_from_maxq_denom_cuda(max_q, denom, query, key, kwargs["thresh"], kwargs["blocksz"])
+            kv_indices, kv_num_indices = mask_utils.packedmask_to_indexmask_cuda(packed, query.shape[2])
         mask_cache.update_cache(current_layer, kv_indices, kv_num_indices)
         return out
     kv_indices, kv_num_indices = mask_cache.get_mask_from_cache(current_layer)
@@ -131,13 +137,14 @@ def blockcached_attn_cuda(query, key, value, current_layer, ditrun, *args, **kwa
     """cached_attn_cuda at the granularity of 64-key blocks (no counterpart in the reference):
     on the refresh steps dense attention with statistics and per-block score maxima, whose threshold
     gives the block lists for q-blocks of ``qblk`` rows (64 or 128, default 128) without a second
-    sweep (``onepass=False``: the bit-packed threshold sweep instead), kept in a
+    sweep (``onepass=False``, or a block-maxima buffer above ``blockmax_budget_bytes`` as in
+    ``cached_attn_cuda``: the bit-packed threshold sweep instead), kept in a
     ``mask_utils.BlockListCache``; on every other step ``sp_attn_block`` over the cached lists in
     their cached work order - one launch."""
     mask_cache = kwargs["mask_cache"]
     qblk = kwargs.get("qblk", 128)
     if mask_cache.run_fullattn(ditrun):
-        if kwargs.get("onepass", True):
+        if mask_utils.use_onepass(query, kwargs.get("onepass"), kwargs.get("blockmax_budget_bytes")):
             # the dense pass also writes the per-(row, key block) score maxima: the lists come from
             # thresholding those, without a second sweep over Q K^T
             out = _out_like(query)

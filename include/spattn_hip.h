@@ -157,27 +157,32 @@ int spattn_booleanmask_to_blocklists(int* blk_indices, int* blk_counts, void* bl
 
 /* Block-level pre-pass without a second score sweep.  The statistics sweeps can also write, next
  * to max_q and denom, the raw score maximum of every row over every 64-key block:
- * blockmax fp32 [batch,heads,Sp/64,Sp] with Sp = 128*ceil(seq/128), entry [J][r] = max over the
- * keys c of block J with c < kv_len of q[r].k[c] (blocks without such a key are not written).
+ * blockmax bf16 [batch,heads,Sp/64,Sp] with Sp = 128*ceil(seq/128), entry [J][r] = max over the
+ * keys c of block J with c < kv_len of q[r].k[c], rounded toward +infinity to bf16 (never below the
+ * fp32 maximum, at most a factor 1 + 2^-7 above it in magnitude; blocks without such a key are not
+ * written): 2*Sp*Sp/64 bytes per head, e.g. 0.81 GB at (1,24,32768), 4.3 GB at (1,24,75856),
+ * 7.2 GB at (1,40,75600).
  * The reference's threshold test  exp2((s[r,c] - max_q[r]) sf) / denom[r] > threshold
  * (include/mask_utils.cuh:231-238) holds for some key of block J exactly when it holds for the
  * block's maximum, so spattn_blockmax_to_blocklists derives the block mask
  *   MB[I,J] = OR_{r in q-block I, r < seq} ( blockmax[J][r] passes the test of row r )
- * and the ascending block lists from 4*Sp*Sp/64 bytes per head instead of the 2*Sp*Sp*D flops of
+ * and the ascending block lists from those bytes instead of the 2*Sp*Sp*D flops of
  * the sweep (include/mask_utils.cuh:131-243 + 273-302 for block-level masks); thresholds can be
- * changed without another sweep.  qblk = 64 or 128 rows per list; outputs as
+ * changed without another sweep.  Because the stored maxima are rounded up, the lists hold every
+ * block of the sweep's block mask and may hold a block whose best key misses the threshold by
+ * less than one bf16 step of its raw score.  qblk = 64 or 128 rows per list; outputs as
  * spattn_packedmask_to_blocklists: blk_indices [batch,heads,ceil(seq/qblk),max_blocks] (entries
  * behind the count keep the caller's fill), blk_counts [batch,heads,ceil(seq/qblk)], optional
  * blockmask uint8 [batch,heads,ceil(seq/qblk),Sp/64].  max_q / denom are those of the same sweep
  * ([batch,heads,1,Sp]); scale and kv_len must be the ones the sweep was given.
  * The _blockmax sweeps replace maxq_denom_impl / attn_maxq_denom_impl
  * (python/extension.cpp:22-33) with the extra output. */
-int spattn_maxq_denom_blockmax(float* max_q, float* denom, float* blockmax, const void* q, const void* k, int batch,
+int spattn_maxq_denom_blockmax(float* max_q, float* denom, void* blockmax, const void* q, const void* k, int batch,
                                int heads, int seq, int D, int kv_len, float scale, void* stream);
-int spattn_fullattn_maxq_denom_blockmax(void* o, float* max_q, float* denom, float* blockmax, const void* q, const void* k,
+int spattn_fullattn_maxq_denom_blockmax(void* o, float* max_q, float* denom, void* blockmax, const void* q, const void* k,
                                         const void* v, int batch, int heads, int seq, int D, int kv_len, float scale,
                                         void* stream);
-int spattn_blockmax_to_blocklists(int* blk_indices, int* blk_counts, void* blockmask, const float* blockmax,
+int spattn_blockmax_to_blocklists(int* blk_indices, int* blk_counts, void* blockmask, const void* blockmax,
                                   const float* max_q, const float* denom, float threshold, int qblk, int batch, int heads,
                                   int seq, int D, int kv_len, float scale, int max_blocks, void* stream);
 
@@ -189,7 +194,9 @@ int spattn_blockmax_to_blocklists(int* blk_indices, int* blk_counts, void* block
  * qblk = 128 for the same statistics, threshold, scale and kv_len - the result is the mask of
  * spattn_booleanmask_128 / spattn_booleanmask_packed (include/mask_utils.cuh:131-243), vote for
  * vote, at the cost of the kept blocks only (about 8 % of the sweep at the density the reference
- * runs at).  A block missing from a list loses its votes; an id outside the row is ignored.
+ * runs at).  A block missing from a list loses its votes; an id outside the row is read as the row's
+ * last pair of key blocks, whose votes are then written as the full sweep would write them (the
+ * result stays within the full sweep's votes).
  * booleanmask / packed, mask_stride, qblk as in the full sweeps (qblk is the row granularity of
  * the bit output; the lists are per 128-row q-block in both cases). */
 int spattn_booleanmask_128_blocks(int* booleanmask, float threshold, int mask_stride, const float* max_q,

@@ -51,6 +51,20 @@ def bf16_round(x: np.ndarray) -> np.ndarray:
     return np.where(np.isfinite(x), out, x)
 
 
+def bf16_round_up(x: np.ndarray) -> np.ndarray:
+    """The smallest bf16 that is not below x (round toward +infinity), returned as fp32; infinities
+    stay.  The form in which the statistics sweeps of this library store their per-block maxima
+    (no counterpart in the reference, whose second sweep recomputes the scores instead).  Pinned
+    in tests/test_oracle.py by the defining property: the result has a bf16 bit pattern, is >= x,
+    and the next bf16 below it is < x."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    u = x.view(np.uint32).astype(np.uint64)
+    neg = (u >> np.uint64(31)) != 0
+    up = np.where(neg, u, u + np.uint64(0xFFFF)) & np.uint64(0xFFFF0000)
+    out = up.astype(np.uint32).view(np.float32)
+    return np.where(np.isfinite(x), out, x)
+
+
 def ceil_div(a: int, b: int) -> int:
     return (a + b - 1) // b
 

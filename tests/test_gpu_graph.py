@@ -22,7 +22,7 @@ def _buffers(dev, B, H, S, D):
     f = dict(device=dev)
     return dict(
         mx=torch.empty((B, H, 1, Sp), **f), dn=torch.empty((B, H, 1, Sp), **f),
-        bmx=torch.empty((B, H, nb, Sp), **f),
+        bmx=torch.empty((B, H, nb, Sp), dtype=torch.bfloat16, **f),
         bi=torch.empty((B, H, SB, nb), dtype=torch.int32, **f), bc=torch.empty((B, H, SB), dtype=torch.int32, **f),
         pk=torch.empty((B, H, SB, Sp // 8), dtype=torch.uint8, **f),
         kvi=torch.empty((B, H, SB, Sp), dtype=torch.int32, **f), kvn=torch.empty((B, H, SB), dtype=torch.int32, **f),

@@ -175,7 +175,7 @@ def test_block_maxima_route_random(dev, seed):
     nb, nkb = Sp // 64, orc.ceil_div(kv, 64)
     mx = torch.full((B, H, 1, Sp), float("nan"), device=dev)
     dn = torch.full((B, H, 1, Sp), float("nan"), device=dev)
-    bmx = torch.full((B, H, nb, Sp), float("nan"), device=dev)
+    bmx = torch.full((B, H, nb, Sp), float("nan"), dtype=torch.bfloat16, device=dev)
     if with_v:
         o = torch.full_like(qd, float("nan"))
         capi.fullattn_maxq_denom_blockmax(o, mx, dn, bmx, qd, kd, vd, kv_len=kv_len)
@@ -186,11 +186,13 @@ def test_block_maxima_route_random(dev, seed):
     wmx, wdn = orc.maxq_denom(f32(q), f32(k), kv_len=kv)
     assert_close_stat(f32(mx), wmx, "max_q", atol=1e-4)
     assert_close_stat(f32(dn), wdn, "denom")
-    got = bmx.cpu().numpy()
+    got = f32(bmx)
     assert np.isnan(got[:, :, nkb:]).all(), "blocks without a key are not written"
     g, w = got[:, :, :nkb, :S], orc.block_row_max(f32(q), f32(k), kv_len=kv)[:, :, :nkb, :S]
-    assert np.isfinite(g).all() and np.all(np.abs(g - w) <= 1e-3 + 1e-4 * np.abs(w))
-    assert np.array_equal(g.max(axis=2), f32(mx).reshape(B, H, Sp)[..., :S])
+    tol = 1e-3 + 1e-4 * np.abs(w)
+    # stored as bf16 rounded up: never below the oracle's maximum, less than one bf16 step above
+    assert np.isfinite(g).all() and np.all(g >= w - tol) and np.all(g <= w + tol + 2.0 ** -7 * np.abs(w))
+    assert np.array_equal(g.max(axis=2), orc.bf16_round_up(f32(mx).reshape(B, H, Sp)[..., :S]))
     dev_bmx = np.nan_to_num(got, nan=-np.inf)
     for qblk in (64, 128):
         nq = orc.ceil_div(S, qblk)
@@ -210,5 +212,9 @@ def test_block_maxima_route_random(dev, seed):
         want_bm, margin = orc.block_mask_from_blockmax(dev_bmx, f32(mx), f32(dn), thr, S, D, qblk=qblk, kv_len=kv)
         near = np.abs(margin) <= 1e-4
         assert np.array_equal(got_bm | near, want_bm | near)
-        band = np.abs(pblk - thr) <= BAND * thr
-        assert np.array_equal(got_bm | band, (pblk > np.float32(thr)) | band)
+        # a superset of the per-key oracle's block mask (the maxima are rounded up), equal outside the band
+        lift = float(np.exp2(2.0 ** -7 * np.abs(dev_bmx[np.isfinite(dev_bmx)]).max() * orc.LOG2E / np.sqrt(D)))
+        exact_bm = pblk > np.float32(thr)
+        band = (pblk >= thr * (1 - BAND) / lift) & (pblk <= thr * (1 + BAND))
+        assert not (exact_bm & ~got_bm & ~band).any()
+        assert np.array_equal(got_bm | band, exact_bm | band)

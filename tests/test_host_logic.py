@@ -156,3 +156,53 @@ def test_topk_mask_definition_takes_the_reference_signature():
     srt = np.sort(sc, axis=-1)
     clear = srt[..., -40] != srt[..., -41]
     assert clear.any() and np.array_equal(got[clear], want[clear])
+
+
+def test_one_sweep_route_is_taken_only_within_the_byte_budget():
+    """The refresh step of the cached functionals takes the one-sweep route when the block-maxima
+    buffer (2 * Sp * Sp / 64 bytes per head) fits the budget, else the reference's two sweeps;
+    onepass=True / False overrides.  Footprints at the shapes the reference compiles."""
+    import torch
+
+    from fgattn_tk_cuda_amd.spattn import mask_utils as mu
+
+    def q_of(B, H, S, D=128):
+        return torch.empty((B, H, S, D), dtype=torch.bfloat16, device="meta")
+
+    assert mu.blockmax_bytes(q_of(1, 24, 32760, 64)) == 2 * 24 * 512 * 32768 == 805306368
+    assert mu.blockmax_bytes(q_of(1, 12, 32768)) == 402653184
+    assert mu.blockmax_bytes(q_of(1, 40, 32760)) == 1342177280
+    assert mu.blockmax_bytes(q_of(1, 12, 75600)) == 2 * 12 * 1182 * 75648
+    assert mu.blockmax_bytes(q_of(1, 24, 75856)) == 2 * 24 * 1186 * 75904 > 4e9
+    assert mu.blockmax_bytes(q_of(1, 40, 75600)) == 2 * 40 * 1182 * 75648 > 7e9
+    assert mu.BLOCKMAX_BUDGET_BYTES == 2 << 30
+    # default budget: cfg 4 and the 32K shapes take one sweep, the 75K shapes with 24 or 40 heads two
+    assert mu.use_onepass(q_of(1, 24, 32760, 64)) and mu.use_onepass(q_of(1, 40, 32760)) and mu.use_onepass(q_of(1, 12, 75600))
+    assert not mu.use_onepass(q_of(1, 24, 75856)) and not mu.use_onepass(q_of(1, 40, 75600))
+    # explicit choices and budgets
+    assert mu.use_onepass(q_of(1, 40, 75600), True) and not mu.use_onepass(q_of(1, 12, 32768), False)
+    assert mu.use_onepass(q_of(1, 40, 75600), None, 8 << 30) and not mu.use_onepass(q_of(1, 12, 32768), None, 1 << 20)
+    assert mu.use_onepass(q_of(1, 12, 32768), None, 402653184) and not mu.use_onepass(q_of(1, 12, 32768), None, 402653183)
+
+
+def test_compressed_list_cache_refuses_ids_that_do_not_fit():
+    """Lists narrower than the sequence (top-k lists): without the sequence length an id beyond the
+    list width is an error instead of a silently dropped key; with it the bits cover the sequence."""
+    import torch
+
+    from fgattn_tk_cuda_amd.spattn import mask_utils as mu
+
+    kvi = torch.full((1, 1, 2, 128), 128, dtype=torch.int32)
+    kvn = torch.tensor([[[3, 2]]], dtype=torch.int32)
+    kvi[0, 0, 0, :3] = torch.tensor([5, 130, 400])
+    kvi[0, 0, 1, :2] = torch.tensor([0, 511])
+    cache = mu.CompressMaskCache([0])
+    with pytest.raises(ValueError):
+        cache.update_cache(0, kvi, kvn)
+    cache.update_cache(0, kvi, kvn, seq_len=500)
+    packed, width, counts = cache.cache[0]
+    assert width == 512 and packed.shape == (1, 1, 2, 64) and counts is kvn
+    bits = mu.unpack(packed)
+    assert bits.shape[-1] == 512
+    assert torch.nonzero(bits[0, 0, 0]).view(-1).tolist() == [5, 130, 400]
+    assert torch.nonzero(bits[0, 0, 1]).view(-1).tolist() == [0, 511]

@@ -447,3 +447,30 @@ def test_qblock_order_is_a_stable_class_sort():
     d = orc.qblock_order(np.full(32, 7))
     assert d[:8].tolist() == [0, 4, 8, 12, 16, 20, 24, 28] and sorted(d.tolist()) == list(range(32))
     assert orc.qblock_order(np.array([1 << 30, 3, 1 << 24, 0])).tolist() == [0, 2, 1, 3]
+
+
+def test_bf16_round_up_by_its_defining_property():
+    """bf16_round_up(x) is the smallest bf16 >= x: it is a bf16 pattern, not below x, and the bf16
+    just below it is below x; bf16 values, zeros and infinities map to themselves."""
+    rng = np.random.default_rng(5)
+    x = np.concatenate([rng.standard_normal(20000).astype(np.float32) * np.float32(40.0),
+                        rng.standard_normal(2000).astype(np.float32) * np.float32(1e-3),
+                        np.array([0.0, -0.0, 1.0, -1.0, 3.140625, -3.140625, np.inf, -np.inf, 1e30, -1e30], np.float32)])
+    y = orc.bf16_round_up(x)
+    yb = y.view(np.uint32)
+    assert np.all((yb & 0xFFFF) == 0), "not a bf16 pattern"
+    assert np.all(y >= x)
+    fin = np.isfinite(x) & (y != 0)
+    # the next bf16 towards -inf: one step of the upper 16 bits (down for positive, up for negative patterns)
+    hi = (yb[fin] >> 16).astype(np.int64)
+    below = np.where(y[fin] > 0, hi - 1, hi + 1).astype(np.uint32) << 16
+    assert np.all(below.view(np.float32) < x[fin])
+    exact = orc.bf16_round(x) == x
+    assert np.array_equal(y[exact], x[exact])
+    assert y[-4] == np.inf and y[-3] == -np.inf
+    # against plain enumeration on a few values: candidates are the two bf16 neighbours
+    for v in x[:200]:
+        lo = np.float32(np.uint32(np.float32(v).view(np.uint32) & 0xFFFF0000).view(np.float32))   # truncation towards zero
+        step = np.float32(np.uint32((np.float32(v).view(np.uint32) & 0xFFFF0000) + 0x10000).view(np.float32))
+        cands = [c for c in (lo, step) if c >= v]
+        assert orc.bf16_round_up(np.array([v], np.float32))[0] == min(cands)
