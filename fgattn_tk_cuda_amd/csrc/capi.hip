@@ -3,6 +3,7 @@
 
 #include <math.h>
 
+#include <atomic>
 #include <mutex>
 
 #include "dispatch.h"
@@ -347,23 +348,33 @@ constexpr int kScratchInts = SPATTN_BALANCED_MAX_QBLOCKS;
 static __device__ __align__(256) int scratch[kScratchInts];
 
 std::mutex g_scratch_mu;
-int* g_scratch_ptr[spattn::kMaxDevices] = {};
+std::atomic<int*> g_scratch_ptr[spattn::kMaxDevices] = {};
 
-// Address of `scratch` on the current device (looked up on the first call per device).
-int scratch_on_current_device(int** out) {
+// Address of `scratch` on the current device.  Looked up on the first call per device (under a
+// lock, and never while `stream` is being captured into a graph: the lookup is a runtime call
+// that may initialise the device's copy of the array); every later call is one atomic load.
+int scratch_on_current_device(int** out, hipStream_t stream) {
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return (int)e;
   if (dev < 0 || dev >= spattn::kMaxDevices) return SPATTN_ERR_SHAPE;
-  std::lock_guard<std::mutex> lock(g_scratch_mu);
-  if (g_scratch_ptr[dev] == nullptr) {
-    void* p = nullptr;
-    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
-    if (e != hipSuccess) return (int)e;
-    if (p == nullptr) return (int)hipErrorInvalidSymbol;
-    g_scratch_ptr[dev] = static_cast<int*>(p);
+  int* known = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (known == nullptr) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (stream != nullptr && hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
+      return SPATTN_ERR_SCRATCH;   // call spattn_init() on this device before recording
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    known = g_scratch_ptr[dev].load(std::memory_order_relaxed);
+    if (known == nullptr) {
+      void* p = nullptr;
+      e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+      if (e != hipSuccess) return (int)e;
+      if (p == nullptr) return (int)hipErrorInvalidSymbol;
+      known = static_cast<int*>(p);
+      g_scratch_ptr[dev].store(known, std::memory_order_release);
+    }
   }
-  *out = g_scratch_ptr[dev];
+  *out = known;
   return SPATTN_OK;
 }
 
@@ -373,7 +384,7 @@ extern "C" {
 
 int spattn_init(void) {
   int* p = nullptr;
-  if (int st = scratch_on_current_device(&p)) return done(st);
+  if (int st = scratch_on_current_device(&p, nullptr)) return done(st);
   // what a first launch would otherwise set on this device: after this call every entry point only launches
   hipError_t e = spattn::prepare_attn_dense();
   if (e == hipSuccess) e = spattn::prepare_attn_blocks();
@@ -392,7 +403,7 @@ int spattn_sp_attn_blocks_balanced(void* o, float* lse, const void* q, const voi
   const long long nq = (long long)B * H * ((S + qblk - 1) / qblk);
   if (nq > kScratchInts) return done(SPATTN_ERR_SCRATCH);
   int* order = nullptr;
-  if (int st = scratch_on_current_device(&order)) return done(st);
+  if (int st = scratch_on_current_device(&order, as_stream(stream))) return done(st);
   // the order kernel writes all nq entries it is asked for: nothing of an earlier call is read
   const hipError_t e = spattn::run_qblock_order(order, blk_counts, (int)nq, as_stream(stream));
   if (e != hipSuccess) return from_hip(e);
@@ -453,7 +464,8 @@ const char* spattn_status_string(int status) {
     case SPATTN_ERR_QBLK: return "q-block must be 64 or 128";
     case SPATTN_ERR_ALIGN: return "pointer is not 16-byte aligned";
     case SPATTN_ERR_SHAPE: return "a size is not positive or is inconsistent";
-    case SPATTN_ERR_SCRATCH: return "more q-blocks than the library's own work-order array holds";
+    case SPATTN_ERR_SCRATCH:
+      return "more q-blocks than the library's own work-order array holds, or its first use on a device inside a stream capture";
     default: return status > 0 ? hipGetErrorString((hipError_t)status) : "unknown status";
   }
 }

@@ -29,7 +29,7 @@ extern "C" {
 #define SPATTN_ERR_QBLK -4       /* q-block is not 64 or 128 */
 #define SPATTN_ERR_ALIGN -5      /* a pointer is not 16-byte aligned */
 #define SPATTN_ERR_SHAPE -6      /* a size is not positive / inconsistent, or seq >= 2^24 */
-#define SPATTN_ERR_SCRATCH -7    /* more q-blocks than SPATTN_BALANCED_MAX_QBLOCKS */
+#define SPATTN_ERR_SCRATCH -7    /* more q-blocks than SPATTN_BALANCED_MAX_QBLOCKS, or first use on a device inside a stream capture */
 
 /* q-blocks (batch * heads * ceil(seq / qblk)) that spattn_sp_attn_blocks_balanced can order */
 #define SPATTN_BALANCED_MAX_QBLOCKS (1 << 20)
@@ -251,7 +251,10 @@ int spattn_sp_attn_blocks_ordered(void* o, float* lse, const void* q, const void
  * spattn_init looks the array's address up for the current device and raises the dynamic-LDS limit
  * of every attention kernel there - the two things a first call on a device otherwise does; it is
  * optional, except that after it every entry point only launches kernels, which is what a caller
- * needs who records his first calls on a device into a HIP graph. */
+ * needs who records his first calls on a device into a HIP graph.  A first call on a device made
+ * while its stream is being captured, without spattn_init before it, returns SPATTN_ERR_SCRATCH
+ * and records nothing (the address lookup is not a call to make inside a capture); a graph that
+ * holds this entry point replays on one stream at a time like the eager calls. */
 int spattn_init(void);
 int spattn_sp_attn_blocks_balanced(void* o, float* lse, const void* q, const void* k, const void* v,
                                    const int* blk_indices, const int* blk_counts, int max_blocks, int qblk, int batch,
