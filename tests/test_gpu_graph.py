@@ -142,3 +142,48 @@ def test_capture_right_after_init_in_a_fresh_process(dev):
     r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=110,
                        cwd=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
     assert r.returncode == 0 and "captured-after-init ok" in r.stdout, r.stdout[-2000:] + r.stderr[-4000:]
+
+
+def test_balanced_entry_point_refuses_its_first_use_inside_a_capture(dev):
+    """A process that records spattn_sp_attn_blocks_balanced into a graph without spattn_init() before: the
+    address of the library's work-order array has not been looked up on the device yet, and the lookup is
+    not made inside a capture - the call returns SPATTN_ERR_SCRATCH and launches nothing; after the capture
+    has ended and spattn_init() has run, the same call works."""
+    print("case balanced first use under capture", flush=True)
+    code = textwrap.dedent("""
+        import ctypes, torch
+        from fgattn_tk_cuda_amd import capi, workloads as wl
+        dev = torch.device("cuda:0")
+        B, H, S, D, qblk = 1, 2, 640, 64, 64
+        q, k, v = (t.to(dev) for t in wl.randn_qkv(B, H, S, D, seed=5))
+        cnt = wl.zipf_counts(B, H, S // qblk, s=1.2, lo=1, hi=S // 64, seed=6)
+        bi, bc = (t.to(dev) for t in wl.ragged_block_lists(B, H, S, qblk, 64, cnt, seed=7))
+        o = torch.full_like(q, float("nan"))
+        lib = capi.load()
+        def call(stream):
+            return lib.spattn_sp_attn_blocks_balanced(o.data_ptr(), None, q.data_ptr(), k.data_ptr(), v.data_ptr(), bi.data_ptr(),
+                                                      bc.data_ptr(), int(bi.shape[3]), qblk, B, H, S, D, 0, ctypes.c_float(0.0), stream)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(g, stream=side):
+                rc = call(side.cuda_stream)
+                # something to record, so that the capture ends as a valid (if useless) graph
+                q2 = q + 0
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        assert rc == -7, rc
+        assert bool(torch.isnan(o.float()).all()), "nothing may have been launched"
+        assert lib.spattn_init() == 0
+        assert call(torch.cuda.current_stream().cuda_stream) == 0
+        torch.cuda.synchronize()
+        e = torch.full_like(q, float("nan"))
+        capi.sp_attn_blocks(e, q, k, v, bi, bc, qblk=qblk)
+        torch.cuda.synchronize()
+        assert torch.equal(o.view(torch.int16), e.view(torch.int16))
+        print("refused-under-capture ok")
+        """)
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=110,
+                       cwd=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    assert r.returncode == 0 and "refused-under-capture ok" in r.stdout, r.stdout[-2000:] + r.stderr[-4000:]
