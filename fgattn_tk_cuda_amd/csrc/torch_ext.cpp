@@ -162,7 +162,8 @@ struct OrderEntry {
   torch::Tensor order;
 };
 static std::mutex g_order_mu;
-static std::vector<OrderEntry> g_orders;
+// never destroyed: the tensors must not be released after the HIP runtime has shut down at process exit
+static std::vector<OrderEntry>& g_orders = *new std::vector<OrderEntry>();
 constexpr size_t kMaxOrderEntries = 1024;
 
 static int64_t counts_version(const torch::Tensor& t) {
