@@ -656,23 +656,23 @@ def main(argv=None) -> int:
             peak_at_clock = PEAK_BF16_TFLOPS * board["gfxclk_mhz"] / 2400.0
             out["roofline"]["at_sustained_clock"] = {"gfxclk_mhz": board["gfxclk_mhz"], "peak": peak_at_clock,
                                                      "frac": tflops / peak_at_clock}
-        # the same launch with every key and value row the same constant: the same instruction stream and
-        # memory traffic with no toggling in the K / V data paths and matrix operands - what the schedule alone
-        # takes when the board is not at its power cap
+        # the same launch with every element of Q, K and V a constant: the same instruction stream and memory
+        # traffic with no toggling in the data paths and matrix operands - what the schedule alone takes when
+        # the board is not at its power cap
         q_, k_, v_, bi_, bc_, o_ = res["tensors"]
-        kc, vc = torch.full_like(k_, 0.25), torch.full_like(v_, 1.0)
+        qc, kc, vc = torch.full_like(q_, 0.5), torch.full_like(k_, 0.25), torch.full_like(v_, 1.0)
         oc = torch.empty_like(o_)
 
         def const_step():
-            capi.sp_attn_blocks(oc, q_, kc, vc, bi_, bc_, qblk=res["qblk"])
+            capi.sp_attn_blocks(oc, qc, kc, vc, bi_, bc_, qblk=res["qblk"])
 
         ms_const, _ = time_steps(const_step, max(2, args.steps // 4), 2)
         board_const = under_load(const_step, ms_const)
-        del kc, vc, oc
+        del qc, kc, vc, oc
         out["board"] = {"during_sp_attn": board, "during_gemm": gm["board"],
-                        "sp_attn_constant_kv": {"ms": ms_const, "tflops": res["flops"] / ms_const / 1e9, "board": board_const,
-                                                "note": "cfg3 launch with K = 0.25 and V = 1 everywhere (Q random): same "
-                                                        "instructions and bytes, no data toggling behind K and V"},
+                        "sp_attn_constant_operands": {"ms": ms_const, "tflops": res["flops"] / ms_const / 1e9, "board": board_const,
+                                                      "note": "cfg3 launch with Q = 0.5, K = 0.25 and V = 1 everywhere: same "
+                                                              "instructions and bytes, no data toggling"},
                         "gemm_bf16_8192_tflops": gm["tflops"], "gemm_mfma_frac": gm["tflops"] / PEAK_BF16_TFLOPS,
                         "sp_attn_vs_gemm": tflops / gm["tflops"],
                         "note": "rocm-smi socket power and graphics clock, three readings each taken right behind a second "
