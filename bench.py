@@ -386,10 +386,12 @@ def bench_cfg4_end_to_end(dev, steps, warmup, seed=0):
     n_sw = max(2, steps // 10)
     ms, _ = time_steps(lambda: capi.fullattn_maxq_denom(o, mx, dn, q, k, v), n_sw, 1)
     dense_flops = 4.0 * B * H * float(S) * S * D
-    out["fullattn_maxq_denom"] = {"ms": ms, "tflops": dense_flops / ms / 1e9, "mfma_frac": dense_flops / ms / 1e9 / PEAK_BF16_TFLOPS}
+    out["fullattn_maxq_denom"] = {"ms": ms, "tflops": dense_flops / ms / 1e9, "mfma_frac": dense_flops / ms / 1e9 / PEAK_BF16_TFLOPS,
+                                  "board": under_load(lambda: capi.fullattn_maxq_denom(o, mx, dn, q, k, v), ms, samples=2)}
     ms, _ = time_steps(lambda: capi.maxq_denom(mx, dn, q, k), n_sw, 1)
     sweep_flops = 2.0 * B * H * float(Sp) * Sp * D
-    out["maxq_denom"] = {"ms": ms, "tflops": sweep_flops / ms / 1e9, "mfma_frac": sweep_flops / ms / 1e9 / PEAK_BF16_TFLOPS}
+    out["maxq_denom"] = {"ms": ms, "tflops": sweep_flops / ms / 1e9, "mfma_frac": sweep_flops / ms / 1e9 / PEAK_BF16_TFLOPS,
+                         "board": under_load(lambda: capi.maxq_denom(mx, dn, q, k), ms, samples=2)}
 
     # threshold: bisection on log(tau) against the kept-block density of the 128-row block mask
     pk = torch.empty((B, H, SB, Sp // 8), dtype=torch.uint8, device=dev)
